@@ -1,4 +1,4 @@
-"""tempura_amd: a small, whole inference engine for decoder-only language models (Llama 3, Mifutar) on one AMD
+"""tempura_amd: a small, whole inference engine for decoder-only language models (Llama 3, Mifutar, Bomotar, Golavik) on one AMD
 MI355X (gfx950).
 
 The names a user starts from (the reference's ``InferenceModel`` and ``inspect``,
@@ -11,9 +11,9 @@ The names a user starts from (the reference's ``InferenceModel`` and ``inspect``
 """
 __version__ = "0.1.0"
 
-from .config import PRESETS, BomotarConfig, LlamaConfig, MifutarConfig, load_config          # noqa: E402,F401
+from .config import PRESETS, BomotarConfig, GolavikConfig, LlamaConfig, MifutarConfig, load_config          # noqa: E402,F401
 from .sampling import SamplingParams                           # noqa: E402,F401
 from .engine import Engine                                     # noqa: E402,F401
 from .inspect import inspect                                   # noqa: E402,F401  (the function, which now hides the module of its name)
 
-__all__ = ["Engine", "SamplingParams", "LlamaConfig", "MifutarConfig", "BomotarConfig", "PRESETS", "load_config", "inspect", "__version__"]
+__all__ = ["Engine", "SamplingParams", "LlamaConfig", "MifutarConfig", "BomotarConfig", "GolavikConfig", "PRESETS", "load_config", "inspect", "__version__"]

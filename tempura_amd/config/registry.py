@@ -14,6 +14,7 @@ from typing import Any, Callable, Dict
 from .llama import ConfigError, LlamaConfig
 from .mifutar import MifutarConfig
 from .bomotar import BomotarConfig
+from .golavik import GolavikConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -74,3 +75,4 @@ register_architecture("LlamaForCausalLM", LlamaConfig)
 register_architecture("llama", LlamaConfig)
 register_architecture("Mifutar", MifutarConfig)
 register_architecture("Bomotar", BomotarConfig)
+register_architecture("Golavik", GolavikConfig)

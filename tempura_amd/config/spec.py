@@ -65,11 +65,14 @@ class LayerCall:
     ``layer`` indexes ``ModelSpec.layers``.  ``cache`` names the cache slot the
     call uses; the first call that names a slot writes it, later calls naming the
     same slot only read it (they compute no keys or values of their own).  When
-    ``cache`` is None the call owns a slot of its own.
+    ``cache`` is None the call owns a slot of its own.  ``before`` names a part of
+    category ``"stream"`` that changes the residual stream right before the call
+    (a learned vector added at the start of a pass over repeated layers, say).
     """
 
     layer: int
     cache: Optional[int] = None
+    before: Optional[PartSpec] = None
 
 
 @dataclass
@@ -103,8 +106,8 @@ class ModelSpec:
             if c.layer < 0 or c.layer >= len(self.layers):
                 raise ValueError(f"run order names layer {c.layer}, model has {len(self.layers)}")
             if c.cache is None:
-                out.append(LayerCall(c.layer, nxt))
+                out.append(LayerCall(c.layer, nxt, c.before))
                 nxt += 1
             else:
-                out.append(LayerCall(c.layer, dense[c.cache]))
+                out.append(LayerCall(c.layer, dense[c.cache], c.before))
         return out

@@ -10,6 +10,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "column_sum.h"
 
 __device__ inline float d_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
 // ln(1 + e^v) without overflow: max(v, 0) + ln(1 + e^-|v|)
@@ -75,19 +76,6 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaArgs a, long pairs
   }
   dot = wave_sum(dot);
   if (lane == 0) a.kq[p] = dot;
-}
-
-// sum over KS neighbouring lanes (from a multiple of KS on); every lane gets it
-template <int KS>
-__device__ inline float column_sum(float v) {
-#define DPP_ADD(ctrl) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xf, 0xf, false))
-  if (KS >= 2) DPP_ADD(0xB1);    // quad_perm [1, 0, 3, 2]
-  if (KS >= 4) DPP_ADD(0x4E);    // quad_perm [2, 3, 0, 1]
-  if (KS >= 8) DPP_ADD(0x141);   // row_half_mirror
-  if (KS >= 16) DPP_ADD(0x140);  // row_mirror
-#undef DPP_ADD
-  if (KS >= 32) v += __shfl_xor(v, 16, TP_WAVE);
-  return v;
 }
 
 template <int PER, int KS>
@@ -302,21 +290,24 @@ extern "C" int tp_delta_scan(float* qkv, int row_stride, const float* decay, con
 // ---- the second product of a low-rank projection ----------------------------------------------
 // out[t, c] = f(sum_i x[t, col0 + i] * wt[i, c]) for a small inner size `rank`; x are float32 rows (the first
 // product's sums), wt float32 [rank, n_out] (the weight transposed, so that neighbouring lanes read neighbouring
-// values).  f: 0 the sum itself; 1 its sigmoid; 2 a decay, exp(-exp(a_log[c / per_head]) * softplus(sum + bias[c])).
+// values).  f: 0 the sum itself; 1 its sigmoid; 2 a decay, exp(-exp(a_log[c / per_head]) * softplus(sum + bias[c]));
+// 3 a decay between exp(-rate) and 1, exp(-rate * sigmoid(sum + bias[c])).  in_act 1: tanh of every x first.
 // A block takes eight rows and 256 columns; a row's sum has the same order of additions wherever the row stands.
 #define LR_ROWS 8
 
 __global__ __launch_bounds__(256) void lowrank_up_kernel(const float* __restrict__ x, int x_stride, int col0, int rank,
                                                          const float* __restrict__ wt, float* __restrict__ out, int n,
                                                          int n_out, int mode, const float* __restrict__ a_log,
-                                                         const float* __restrict__ bias, int per_head) {
+                                                         const float* __restrict__ bias, int per_head, int in_act,
+                                                         float rate_const) {
   // (blocks of 64 or 256 threads: a thread owns one column)
   extern __shared__ __attribute__((aligned(16))) float xs[];   // [LR_ROWS][rank4]: rows padded with zeros to four
   const int rank4 = (rank + 3) & ~3;
   const int t0 = blockIdx.x * LR_ROWS, c = blockIdx.y * blockDim.x + threadIdx.x;
   for (int idx = threadIdx.x; idx < LR_ROWS * rank4; idx += blockDim.x) {
     const int t = idx / rank4, i = idx % rank4;
-    xs[idx] = (t0 + t < n && i < rank) ? x[(size_t)(t0 + t) * x_stride + col0 + i] : 0.f;
+    const float v = (t0 + t < n && i < rank) ? x[(size_t)(t0 + t) * x_stride + col0 + i] : 0.f;
+    xs[idx] = in_act == 1 ? tanhf(v) : v;
   }
   __syncthreads();
   if (c >= n_out) return;
@@ -342,21 +333,27 @@ __global__ __launch_bounds__(256) void lowrank_up_kernel(const float* __restrict
     rate = expf(a_log[c / per_head]);
     b = bias[c];
   }
+  if (mode == 3) {
+    rate = rate_const;
+    b = bias[c];
+  }
 #pragma unroll
   for (int t = 0; t < LR_ROWS; ++t) {
     if (t0 + t >= n) break;
     float v = acc[t];
     if (mode == 1) v = d_sigmoid(v);
     if (mode == 2) v = expf(-rate * d_softplus(v + b));
+    if (mode == 3) v = expf(-rate * d_sigmoid(v + b));
     out[(size_t)(t0 + t) * n_out + c] = v;
   }
 }
 
 extern "C" int tp_lowrank_up(const float* x, int x_stride, int col0, int rank, const float* wt, float* out, int n, int n_out,
-                             int mode, const float* a_log, const float* bias, int per_head, hipStream_t s) {
+                             int mode, const float* a_log, const float* bias, int per_head, int in_act, float rate, hipStream_t s) {
   TP_REQUIRE(n >= 0 && rank > 0 && n_out > 0 && col0 >= 0 && x_stride >= col0 + rank, "lowrank_up: bad sizes");
   TP_REQUIRE(rank <= 1024, "lowrank_up: inner size %d exceeds 1024", rank);
-  TP_REQUIRE(mode >= 0 && mode <= 2, "lowrank_up: unknown epilogue %d", mode);
+  TP_REQUIRE(mode >= 0 && mode <= 3 && (in_act == 0 || in_act == 1), "lowrank_up: unknown epilogue %d or input function %d", mode, in_act);
+  TP_REQUIRE(mode != 3 || bias, "lowrank_up: the decay needs its biases");
   TP_REQUIRE(mode != 2 || (a_log && bias && per_head > 0), "lowrank_up: the decay needs its rates and biases");
   if (n == 0) return 0;
   // (a few rows: blocks of one wave, so that the columns are spread over many CUs)
@@ -364,19 +361,21 @@ extern "C" int tp_lowrank_up(const float* x, int x_stride, int col0, int rank, c
   const dim3 grid((n + LR_ROWS - 1) / LR_ROWS, (n_out + threads - 1) / threads);
   TP_REQUIRE(grid.y <= 65535, "lowrank_up: too many columns");
   hipLaunchKernelGGL(lowrank_up_kernel, grid, dim3(threads), sizeof(float) * LR_ROWS * ((rank + 3) & ~3), s, x, x_stride, col0, rank, wt, out, n,
-                     n_out, mode, a_log, bias, per_head);
+                     n_out, mode, a_log, bias, per_head, in_act, rate);
   TP_CHECK_LAUNCH("lowrank_up");
   return 0;
 }
 
 // ---- norm per head with a gate ----------------------------------------------------------------
 // out[t, out_col0 + h * vdim + d] = o[t, h, d] / sqrt(mean_d o^2 + eps) * w[d] * gate[t, h * vdim + d] * scale;
-// gate (float32, already between 0 and 1) may be missing.  One wave per (token, head).
+// gate (float32, already between 0 and 1) may be missing.  w_stride vdim: every head has its own weight [heads, vdim]
+// (0: one weight [vdim] for all).  gate_raw: the gate is sigmoid(gate[t * gate_stride + h * vdim + d]) of raw rows.
+// One wave per (token, head).
 template <typename TO>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                              const float* __restrict__ gate, float eps, float scale,
                                                              TO* __restrict__ out, int out_stride, int out_col0, long pairs,
-                                                             int heads, int vdim) {
+                                                             int heads, int vdim, int w_stride, size_t gate_stride, int gate_raw) {
   const long p = (long)blockIdx.x * 4 + threadIdx.x / TP_WAVE;
   const int lane = threadIdx.x % TP_WAVE;
   if (p >= pairs) return;
@@ -388,15 +387,18 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   ss = wave_sum(ss);
   const float rstd = 1.0f / sqrtf(ss / (float)vdim + eps);
   TO* dst = out + (size_t)t * out_stride + out_col0 + (size_t)h * vdim;
+  const float* wh = w + (size_t)h * w_stride;
+  const float* gr = gate != nullptr ? gate + (size_t)t * gate_stride + (size_t)h * vdim : nullptr;
   for (int d = lane; d < vdim; d += TP_WAVE) {
-    float v = row[d] * rstd * w[d];
-    if (gate != nullptr) v *= gate[(size_t)p * vdim + d];
+    float v = row[d] * rstd * wh[d];
+    if (gr != nullptr) v *= gate_raw ? d_sigmoid(gr[d]) : gr[d];
     from_float(dst + d, v * scale);
   }
 }
 
 extern "C" int tp_head_norm_gate(const float* o, const float* w, const float* gate, float eps, float scale, void* out, int out_dt,
-                                 int out_stride, int out_col0, int n, int heads, int vdim, hipStream_t s) {
+                                 int out_stride, int out_col0, int n, int heads, int vdim, int w_per_head, size_t gate_stride,
+                                 int gate_raw, hipStream_t s) {
   TP_REQUIRE(n >= 0 && heads > 0 && vdim > 0 && out_col0 >= 0 && out_stride >= out_col0 + heads * vdim, "head_norm_gate: bad sizes");
   if (n == 0) return 0;
   const long pairs = (long)n * heads;
@@ -404,10 +406,10 @@ extern "C" int tp_head_norm_gate(const float* o, const float* w, const float* ga
   TP_REQUIRE(blocks < 0x7fffffffL, "head_norm_gate: too many rows");
   if (out_dt == TP_F32)
     hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3((unsigned)blocks), dim3(256), 0, s, o, w, gate, eps, scale, (float*)out,
-                       out_stride, out_col0, pairs, heads, vdim);
+                       out_stride, out_col0, pairs, heads, vdim, w_per_head ? vdim : 0, gate_stride, gate_raw);
   else if (out_dt == TP_BF16)
     hipLaunchKernelGGL(head_norm_gate_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, s, o, w, gate, eps, scale, (bf16_t*)out,
-                       out_stride, out_col0, pairs, heads, vdim);
+                       out_stride, out_col0, pairs, heads, vdim, w_per_head ? vdim : 0, gate_stride, gate_raw);
   else
     TP_REQUIRE(false, "head_norm_gate: unknown dtype %d", out_dt);
   TP_CHECK_LAUNCH("head_norm_gate");

@@ -329,10 +329,15 @@ __device__ inline void wave_arg_best(float& v, int& i) {
   }
 }
 
+// score_kind 0: s = softmax over the experts; 1: s = sigmoid of each logit by itself.  The choice score is s plus the
+// correction (none: s).  A group is ranked by the sum of its `group_best` largest choice scores.  The weights are the
+// chosen experts' s, with `normalize` divided by their sum plus sum_eps (added in the order of choice), times `scale`.
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int logit_stride,
                                                         const float* __restrict__ correction, int experts, int top,
                                                         int groups, int keep, float* __restrict__ dense,
-                                                        int* __restrict__ ids, float* __restrict__ weights, int n) {
+                                                        int* __restrict__ ids, float* __restrict__ weights, int n,
+                                                        int score_kind, int group_best, int normalize, float sum_eps,
+                                                        float scale) {
   extern __shared__ float lds[];   // per wave: choice scores [experts], then group scores [groups]
   const int wave = threadIdx.x / TP_WAVE, lane = threadIdx.x % TP_WAVE;
   // (a wave past the last token works on the last token again and stores nothing: every wave reaches every barrier)
@@ -341,27 +346,35 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
   float* choice_l = lds + (size_t)wave * (experts + max(groups, 1));
   float* group_l = choice_l + experts;
   float z[ROUTE_PER_LANE], sc[ROUTE_PER_LANE], ch[ROUTE_PER_LANE];
+  int won[ROUTE_PER_LANE];
   float mx = -INFINITY;
 #pragma unroll
   for (int k = 0; k < ROUTE_PER_LANE; ++k) {
     const int e = lane + k * TP_WAVE;
     z[k] = e < experts ? logits[(size_t)t * logit_stride + e] : -INFINITY;
     mx = fmaxf(mx, z[k]);
+    won[k] = -1;
   }
-  mx = wave_max(mx);
-  float sum = 0.f;
+  if (score_kind == 1) {
 #pragma unroll
-  for (int k = 0; k < ROUTE_PER_LANE; ++k) {
-    sc[k] = lane + k * TP_WAVE < experts ? expf(z[k] - mx) : 0.f;
-    sum += sc[k];
+    for (int k = 0; k < ROUTE_PER_LANE; ++k) sc[k] = lane + k * TP_WAVE < experts ? l_sigmoid(z[k]) : 0.f;
+  } else {
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+      sc[k] = lane + k * TP_WAVE < experts ? expf(z[k] - mx) : 0.f;
+      sum += sc[k];
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int k = 0; k < ROUTE_PER_LANE; ++k) sc[k] *= inv;
   }
-  sum = wave_sum(sum);
-  const float inv = 1.0f / sum;
 #pragma unroll
   for (int k = 0; k < ROUTE_PER_LANE; ++k) {
     const int e = lane + k * TP_WAVE;
-    sc[k] *= inv;
-    ch[k] = e < experts ? sc[k] + correction[e] : -INFINITY;
+    ch[k] = e < experts ? (correction != nullptr ? sc[k] + correction[e] : sc[k]) : -INFINITY;
     if (e < experts) {
       choice_l[e] = ch[k];
       if (live) dense[(size_t)t * experts + e] = 0.f;
@@ -371,9 +384,25 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     const int per = experts / groups;
     __syncthreads();
     for (int g = lane; g < groups; g += TP_WAVE) {
-      float best = -INFINITY;
-      for (int i = 0; i < per; ++i) best = fmaxf(best, choice_l[g * per + i]);
-      group_l[g] = best;
+      // the group's largest scores one after the other (equal scores: the lower index first), added in that order
+      float total = 0.f, pv = INFINITY;
+      int pi = -1;
+      for (int b = 0; b < group_best; ++b) {
+        float best = -INFINITY;
+        int bi = -1;
+        for (int i = 0; i < per; ++i) {
+          const float v = choice_l[g * per + i];
+          if ((v < pv || (v == pv && i > pi)) && (bi < 0 || v > best)) {
+            best = v;
+            bi = i;
+          }
+        }
+        if (bi < 0) break;
+        total = b == 0 ? best : total + best;
+        pv = best;
+        pi = bi;
+      }
+      group_l[g] = total;
     }
     __syncthreads();
     // the `keep` best groups, one after the other; a kept group's score becomes +inf as its mark
@@ -398,6 +427,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
       if (e < experts && group_l[e / per] != INFINITY) ch[k] = -INFINITY;
     }
   }
+  float chosen_sum = 0.f;
   for (int it = 0; it < top; ++it) {
     float bv = -INFINITY, bs = 0.f;
     int bi = 0x7fffffff, bk = -1;
@@ -415,29 +445,41 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     int i = bi;
     wave_arg_best(v, i);
     if (i == 0x7fffffff) break;   // fewer allowed experts than `top` (uniform over the wave)
+    chosen_sum += __shfl(bs, i % TP_WAVE, TP_WAVE);   // (the winner's lane holds its score; every lane adds alike)
     if (i == bi && bk >= 0) {
       // this lane owns the winner
 #pragma unroll
       for (int k = 0; k < ROUTE_PER_LANE; ++k)
-        if (k == bk) ch[k] = -INFINITY;
-      if (live) {
-        dense[(size_t)t * experts + i] = bs;
-        ids[(size_t)t * top + it] = i;
-        weights[(size_t)t * top + it] = bs;
-      }
+        if (k == bk) {
+          ch[k] = -INFINITY;
+          won[k] = it;
+        }
+    }
+  }
+  const float factor = normalize ? scale / (chosen_sum + sum_eps) : scale;
+#pragma unroll
+  for (int k = 0; k < ROUTE_PER_LANE; ++k) {
+    if (won[k] >= 0 && live) {
+      const int e = lane + k * TP_WAVE;
+      const float w = (normalize || scale != 1.0f) ? sc[k] * factor : sc[k];
+      dense[(size_t)t * experts + e] = w;
+      ids[(size_t)t * top + won[k]] = e;
+      weights[(size_t)t * top + won[k]] = w;
     }
   }
 }
 
 extern "C" int tp_moe_route(const float* logits, int logit_stride, const float* correction, int experts, int top, int groups,
-                            int keep, float* dense, int* ids, float* weights, int n, hipStream_t s) {
+                            int keep, float* dense, int* ids, float* weights, int n, int score_kind, int group_best,
+                            int normalize, float sum_eps, float scale, hipStream_t s) {
   TP_REQUIRE(n >= 0 && experts > 0 && top > 0 && top <= experts && logit_stride >= experts, "moe_route: bad sizes");
   TP_REQUIRE(experts <= TP_WAVE * ROUTE_PER_LANE, "moe_route: %d experts exceed %d", experts, TP_WAVE * ROUTE_PER_LANE);
   TP_REQUIRE(groups <= 1 || (experts % groups == 0 && keep >= 1 && keep <= groups), "moe_route: bad groups");
+  TP_REQUIRE((score_kind == 0 || score_kind == 1) && group_best >= 1, "moe_route: bad score kind or group_best");
   if (n == 0) return 0;
   const size_t shmem = sizeof(float) * 4 * (size_t)(experts + (groups > 1 ? groups : 1));
   hipLaunchKernelGGL(moe_route_kernel, dim3((n + 3) / 4), dim3(256), shmem, s, logits, logit_stride, correction, experts, top, groups,
-                     keep, dense, ids, weights, n);
+                     keep, dense, ids, weights, n, score_kind, group_best, normalize, sum_eps, scale);
   TP_CHECK_LAUNCH("moe_route");
   return 0;
 }
@@ -559,5 +601,170 @@ extern "C" int tp_moe_spread(const void* a, int dt, const float* dense, void* ou
   else
     TP_REQUIRE(false, "moe_spread: unknown dtype %d", dt);
   TP_CHECK_LAUNCH("moe_spread");
+  return 0;
+}
+
+// ---- RMS norm in equal parts of a run of columns ----------------------------------------------
+// The `width` columns from col0 on of float32 rows [*, x_stride] are split into `groups` equal consecutive parts;
+// each part is divided by its own sqrt(mean(part^2) + eps) and the whole multiplied by w [width].  `rows` (optional)
+// picks the input row of each output row; out [n_out, width].  One block per output row, a wave per part in turn.
+template <typename TO>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* __restrict__ x, size_t x_stride, int col0,
+                                                            const float* __restrict__ w, const int* __restrict__ rows,
+                                                            TO* __restrict__ out, int width, int groups, float eps) {
+  const int r = blockIdx.x;
+  const float* xr = x + (size_t)(rows ? rows[r] : r) * x_stride + col0;
+  TO* o = out + (size_t)r * width;
+  const int wave = threadIdx.x / TP_WAVE, lane = threadIdx.x % TP_WAVE, waves = blockDim.x / TP_WAVE;
+  const int per = width / groups;
+  for (int g = wave; g < groups; g += waves) {
+    const float* p = xr + (size_t)g * per;
+    float ss = 0.f;
+    for (int i = lane; i < per; i += TP_WAVE) ss = fmaf(p[i], p[i], ss);
+    ss = wave_sum(ss);
+    const float scale = 1.0f / sqrtf(ss / (float)per + eps);
+    for (int i = lane; i < per; i += TP_WAVE) from_float(o + (size_t)g * per + i, p[i] * scale * w[(size_t)g * per + i]);
+  }
+}
+
+extern "C" int tp_group_rmsnorm(const float* x, size_t x_stride, int col0, const float* w, const int* rows, void* out, int out_dt,
+                                int n_out, int width, int groups, float eps, hipStream_t s) {
+  TP_REQUIRE(n_out >= 0 && width > 0 && groups > 0 && width % groups == 0 && col0 >= 0 && x_stride >= (size_t)col0 + width,
+             "group_rmsnorm: bad sizes");
+  if (n_out == 0) return 0;
+  const int threads = groups >= 4 ? 256 : (groups * TP_WAVE);
+  if (out_dt == TP_F32)
+    hipLaunchKernelGGL(group_rmsnorm_kernel<float>, dim3(n_out), dim3(threads), 0, s, x, x_stride, col0, w, rows, (float*)out, width, groups, eps);
+  else if (out_dt == TP_BF16)
+    hipLaunchKernelGGL(group_rmsnorm_kernel<bf16_t>, dim3(n_out), dim3(threads), 0, s, x, x_stride, col0, w, rows, (bf16_t*)out, width, groups, eps);
+  else
+    TP_REQUIRE(false, "group_rmsnorm: unknown dtype %d", out_dt);
+  TP_CHECK_LAUNCH("group_rmsnorm");
+  return 0;
+}
+
+// ---- what sublayers read of normed rows: the rows plus a short convolution of them over time ---
+// x float32 [n, width]; w [subs, taps, width] (tap-major; the last tap is the current token's).  For sublayer s:
+// out_s[t, c] = x[t, c] + sum_k w[s, k, c] * x[t - (taps - 1 - k), c], the rows before a run's first token coming from
+// the request's state row (from element state_off on: [taps - 1, width], oldest first; zeros for a fresh request).
+// The sublayers read the same rows, so one state serves them all; a second kernel leaves the run's last rows there.
+template <typename TO>
+__global__ void residual_conv_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ state,
+                                     size_t state_stride, size_t state_off, const int* __restrict__ cu_seqlens,
+                                     const int* __restrict__ token_req, const int* __restrict__ state_slots, TO* __restrict__ out,
+                                     size_t out_stride_sub, int width, int taps, int subs, int channel_blocks) {
+  const int t = blockIdx.x / channel_blocks;
+  const int c = (blockIdx.x % channel_blocks) * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int r = token_req[t];
+  const int start = cu_seqlens[r];
+  const int i = t - start;
+  const float* st = state + (size_t)state_slots[r] * state_stride + state_off;
+  const float cur = x[(size_t)t * width + c];
+  for (int sub = 0; sub < subs; ++sub) {
+    float acc = 0.f;
+    for (int k = 0; k < taps; ++k) {
+      const int src = i - (taps - 1 - k);
+      const float v = src >= 0 ? x[(size_t)(start + src) * width + c] : st[(size_t)(taps - 1 + src) * width + c];
+      acc = fmaf(w[((size_t)sub * taps + k) * width + c], v, acc);
+    }
+    from_float(out + (size_t)sub * out_stride_sub + (size_t)t * width + c, cur + acc);
+  }
+}
+
+__global__ void residual_conv_state_kernel(const float* __restrict__ x, float* __restrict__ state, size_t state_stride,
+                                           size_t state_off, const int* __restrict__ cu_seqlens,
+                                           const int* __restrict__ state_slots, int width, int taps) {
+  const int r = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int start = cu_seqlens[r], len = cu_seqlens[r + 1] - start;
+  if (len <= 0) return;
+  float* st = state + (size_t)state_slots[r] * state_stride + state_off;
+  // in place, ascending: entry j takes entry j + len of the old state or a row of the run; entries below j are never read again
+  for (int j = 0; j < taps - 1; ++j) {
+    const int src = len - (taps - 1) + j;
+    st[(size_t)j * width + c] = src >= 0 ? x[(size_t)(start + src) * width + c] : st[(size_t)(j + len) * width + c];
+  }
+}
+
+extern "C" int tp_residual_conv(const float* x, const float* w, float* state, size_t state_stride, size_t state_off,
+                                const int* cu_seqlens, const int* token_req, const int* state_slots, void* out, int out_dt, int n,
+                                int n_req, int width, int taps, int subs, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && n_req >= 0 && width > 0 && taps >= 1 && subs >= 1, "residual_conv: bad sizes");
+  TP_REQUIRE(state_stride >= state_off + (size_t)(taps - 1) * width, "residual_conv: state rows too short");
+  if (n == 0) return 0;
+  const int threads = width >= 256 ? 256 : 64;
+  const int cb = (width + threads - 1) / threads;
+  TP_REQUIRE(cb <= 65535 && (long)n * cb < 0x7fffffffL, "residual_conv: too many channels or tokens");
+  const size_t sub_stride = (size_t)n * width;
+  if (out_dt == TP_F32)
+    hipLaunchKernelGGL(residual_conv_kernel<float>, dim3((unsigned)((long)n * cb)), dim3(threads), 0, s, x, w, state, state_stride,
+                       state_off, cu_seqlens, token_req, state_slots, (float*)out, sub_stride, width, taps, subs, cb);
+  else if (out_dt == TP_BF16)
+    hipLaunchKernelGGL(residual_conv_kernel<bf16_t>, dim3((unsigned)((long)n * cb)), dim3(threads), 0, s, x, w, state, state_stride,
+                       state_off, cu_seqlens, token_req, state_slots, (bf16_t*)out, sub_stride, width, taps, subs, cb);
+  else
+    TP_REQUIRE(false, "residual_conv: unknown dtype %d", out_dt);
+  if (taps > 1 && n_req > 0)
+    hipLaunchKernelGGL(residual_conv_state_kernel, dim3(n_req, cb), dim3(threads), 0, s, x, state, state_stride, state_off, cu_seqlens,
+                       state_slots, width, taps);
+  TP_CHECK_LAUNCH("residual_conv");
+  return 0;
+}
+
+// ---- one row of a table added to every row of the stream --------------------------------------
+__global__ void add_row_kernel(float* __restrict__ h, const float* __restrict__ row, size_t total, int width) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) h[i] += row[i % width];
+}
+
+extern "C" int tp_add_row(float* h, const float* row, int n, int width, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && width > 0, "add_row: bad sizes");
+  if (n == 0) return 0;
+  const size_t total = (size_t)n * width;
+  TP_REQUIRE((total + 255) / 256 < 0x7fffffffUL, "add_row: too many elements");
+  hipLaunchKernelGGL(add_row_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, h, row, total, width);
+  TP_CHECK_LAUNCH("add_row");
+  return 0;
+}
+
+// ---- rows of q | k | v for an attention whose keys and values are expanded from a latent --------
+// Per token: q [heads, key] comes from the projection's rows as it stands (key = rot + dim elements a head, the
+// rotated ones first); head h's key is the ONE shared rotated part (rot elements of the projection's rows, not yet
+// rotated) followed by its own dim unrotated elements of the expansion `up` ([heads * dim | heads * vdim] a row);
+// its value the head's vdim elements of `up`.  out [n, 2 * heads * key + heads * vdim] float32, the layout the
+// rotation-and-store kernel takes.
+__global__ void latent_rows_kernel(const float* __restrict__ proj, size_t proj_stride, int q_col0, int rot_col0,
+                                   const float* __restrict__ up, size_t up_stride, float* __restrict__ out, int heads, int dim,
+                                   int rot, int vdim) {
+  const int t = blockIdx.x;
+  const int key = rot + dim, qk = heads * key, width = 2 * qk + heads * vdim;
+  const float* pr = proj + (size_t)t * proj_stride;
+  const float* ur = up + (size_t)t * up_stride;
+  float* o = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v;
+    if (i < qk) {
+      v = pr[q_col0 + i];
+    } else if (i < 2 * qk) {
+      const int h = (i - qk) / key, d = (i - qk) % key;
+      v = d < rot ? pr[rot_col0 + d] : ur[h * dim + d - rot];
+    } else {
+      v = ur[heads * dim + i - 2 * qk];
+    }
+    o[i] = v;
+  }
+}
+
+extern "C" int tp_latent_rows(const float* proj, size_t proj_stride, int q_col0, int rot_col0, const float* up, size_t up_stride,
+                              float* out, int n, int heads, int dim, int rot, int vdim, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && heads > 0 && dim > 0 && rot >= 0 && vdim > 0 && q_col0 >= 0 && rot_col0 >= 0, "latent_rows: bad sizes");
+  TP_REQUIRE(proj_stride >= (size_t)q_col0 + (size_t)heads * (rot + dim) && proj_stride >= (size_t)rot_col0 + rot &&
+                 up_stride >= (size_t)heads * (dim + vdim), "latent_rows: rows too short");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(latent_rows_kernel, dim3(n), dim3(256), 0, s, proj, proj_stride, q_col0, rot_col0, up, up_stride, out, heads, dim,
+                     rot, vdim);
+  TP_CHECK_LAUNCH("latent_rows");
   return 0;
 }

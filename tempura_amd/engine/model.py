@@ -35,6 +35,8 @@ class CausalLM:
         self.final_norm = build_part("norm", spec.final_norm, h, dtype, device)
         self.lm_head = part_class("lm_head", spec.lm_head.kind)(spec.lm_head, h, dtype, device, spec.vocab_size)
         self.order = spec.resolved_order()
+        #: per run-order entry: the part that changes the residual stream right before the call, or None
+        self.before = [None if c.before is None else build_part("stream", c.before, h, dtype, device) for c in self.order]
         #: copies of the residual stream that the blocks keep side by side; ``h`` is [tokens, streams * hidden]
         self.streams = int(getattr(spec, "streams", 1) or 1)
         #: None, or a callable (i, h) called before run-order entry i and once after the last with the residual
@@ -108,6 +110,9 @@ class CausalLM:
         self.embedding.load_weights(get)
         for layer in self.layers:
             layer.load_weights(get)
+        for part in self.before:
+            if part is not None:
+                part.load_weights(get)
         self.final_norm.load_weights(get)
         self.lm_head.load_weights(get, self.embedding)
 
@@ -128,7 +133,7 @@ class CausalLM:
                 if store.data_ptr() not in seen:
                     seen.add(store.data_ptr())
                     total += store.nbytes()
-        objs = [self.final_norm, self.lm_head]
+        objs = [self.final_norm, self.lm_head] + [p for p in self.before if p is not None]
         if include_embedding:
             objs.append(self.embedding)
         for layer in self.layers:
@@ -162,6 +167,9 @@ class CausalLM:
             if observe is not None:
                 observe(i, self._stream_sum(h))
             layer = self.layers[call.layer]
+            if self.before[i] is not None:
+                self.before[i].forward(h, ctx)
+                x = None      # (rows handed over by the block before were normed from the stream as it was)
             if not hasattr(layer, "entry_norm"):
                 layer.forward(h, ctx, caches[i])
                 x = None
@@ -169,6 +177,8 @@ class CausalLM:
             after = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else None
             # (a block hands rows only to a block of its own kind: the two agree on what is handed over)
             same = hasattr(after, "entry_norm") and getattr(after, "handoff", None) == getattr(layer, "handoff", None)
+            if i + 1 < len(self.order) and self.before[i + 1] is not None:
+                same = False      # (the stream changes between the two blocks: nothing is handed over)
             next_norm = after.entry_norm(m) if same else None
             x = layer.forward(h, ctx, caches[i], x, next_norm)
         if observe is not None:
@@ -176,7 +186,7 @@ class CausalLM:
         if self.streams > 1:
             # the final norm reads the sum of the copies, at the wanted rows only
             norm = self.final_norm
-            if type(norm).__name__ == "RMSNorm":
+            if type(norm).__name__ == "RMSNorm" and getattr(norm, "groups", 1) == 1:
                 x = ops.stream_step(h, self.streams, norm_weight=norm.weight, eps=norm.eps, out_dtype=self.dtype,
                                     rows=ctx.logit_rows, write_back=False)
             else:

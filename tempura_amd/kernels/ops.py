@@ -372,9 +372,12 @@ def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_col0: int, weight: t
 
 
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
-            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """float32 [n, hidden] -> out_dtype [n or len(rows), hidden]."""
+            rows: Optional[torch.Tensor] = None, groups: int = 1) -> torch.Tensor:
+    """float32 [n, hidden] -> out_dtype [n or len(rows), hidden].  ``groups`` > 1: the row is split into that many
+    equal consecutive parts and each is divided by its own root mean square."""
     if _backend is not None:
+        if groups != 1:
+            return _backend.rmsnorm(h, weight, eps, out_dtype, rows, groups)
         return _backend.rmsnorm(h, weight, eps, out_dtype, rows)
     _dev_ok(h, weight, rows)
     _need(h.dtype == torch.float32 and h.dim() == 2, "rmsnorm: input must be float32 [n, hidden]")
@@ -384,6 +387,11 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
         n_out = rows.numel()
         _i32(rows, n_out, "rmsnorm rows") if n_out else None
     out = torch.empty((n_out, h.shape[1]), dtype=out_dtype, device=h.device)
+    if groups != 1:
+        _need(groups > 0 and h.shape[1] % groups == 0, "rmsnorm: groups must divide the row")
+        _call("tp_group_rmsnorm", _ptr(h), ctypes.c_size_t(h.shape[1]), 0, _ptr(weight), _ptr(rows), _ptr(out), _dtcode(out_dtype),
+              n_out, h.shape[1], int(groups), ctypes.c_float(eps), _stream())
+        return out
     _call("tp_rmsnorm", _ptr(h), _ptr(weight), _ptr(rows), _ptr(out), _dtcode(out_dtype), n_out, h.shape[1],
           ctypes.c_float(eps), _stream())
     return out
@@ -1264,34 +1272,49 @@ def activation(u: torch.Tensor, kind: str, out_dtype: torch.dtype) -> torch.Tens
     return out
 
 
-def moe_route(logits: torch.Tensor, correction: torch.Tensor, experts: int, top: int, groups: int, keep: int):
-    """Router of a mixture of experts over float32 logits [n, >= experts]: s = softmax over the experts; an expert's
-    choice score is s + correction; with ``groups`` > 1 only the experts of the ``keep`` groups (of neighbours) with
-    the largest best choice score can be chosen; the ``top`` best allowed experts are chosen and weigh s.  Returns
-    (dense float32 [n, experts] with a chosen expert's weight and 0 elsewhere, ids int32 [n, top], weights [n, top])."""
+ROUTE_SCORES = {"softmax": 0, "sigmoid": 1}
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, groups: int, keep: int,
+              score: str = "softmax", group_best: int = 1, normalize: bool = False, sum_eps: float = 0.0, scale: float = 1.0):
+    """Router of a mixture of experts over float32 logits [n, >= experts]: s = softmax over the experts (``score``
+    ``"sigmoid"``: the sigmoid of each logit by itself); an expert's choice score is s + correction (None: s); with
+    ``groups`` > 1 only the experts of the ``keep`` groups (of neighbours) whose ``group_best`` largest choice scores
+    add up highest can be chosen; the ``top`` best allowed experts are chosen and weigh s, with ``normalize`` divided by
+    the chosen experts' sum (+ ``sum_eps``), times ``scale``.  Returns (dense float32 [n, experts] with a chosen expert's
+    weight and 0 elsewhere, ids int32 [n, top], weights [n, top])."""
+    _need(score in ROUTE_SCORES, f"moe_route: score {score!r} unknown")
     if _backend is not None:
-        return _backend.moe_route(logits, correction, experts, top, groups, keep)
+        if (score, group_best, normalize, scale) == ("softmax", 1, False, 1.0) and correction is not None:
+            return _backend.moe_route(logits, correction, experts, top, groups, keep)
+        return _backend.moe_route(logits, correction, experts, top, groups, keep, score, group_best, normalize, sum_eps, scale)
     _dev_ok(logits, correction)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] >= experts, "moe_route: logits must be float32 [n, experts]")
-    _need(correction.dtype == torch.float32 and correction.numel() == experts, "moe_route: correction must be float32 [experts]")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == experts), "moe_route: correction must be float32 [experts]")
+    _need(group_best >= 1, "moe_route: group_best must be at least 1")
     n = logits.shape[0]
     dense = torch.empty((n, experts), dtype=torch.float32, device=logits.device)
     ids = torch.empty((n, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=logits.device)
     _call("tp_moe_route", _ptr(logits), logits.shape[1], _ptr(correction), int(experts), int(top), int(groups), int(keep), _ptr(dense),
-          _ptr(ids), _ptr(weights), n, _stream())
+          _ptr(ids), _ptr(weights), n, ROUTE_SCORES[score], int(group_best), int(bool(normalize)), ctypes.c_float(sum_eps),
+          ctypes.c_float(scale), _stream())
     return dense, ids, weights
 
 
-LOWRANK_MODES = {"plain": 0, "sigmoid": 1, "decay": 2}
+LOWRANK_MODES = {"plain": 0, "sigmoid": 1, "decay": 2, "rate_sigmoid": 3}
 
 
 def lowrank_up(x: torch.Tensor, col0: int, weight_t: torch.Tensor, mode: str = "plain", a_log: Optional[torch.Tensor] = None,
-               bias: Optional[torch.Tensor] = None, per_head: int = 0) -> torch.Tensor:
-    """The second product of a low-rank projection: float32 [n, N] = f(x[:, col0: col0 + r] @ weight_t), ``x`` float32
+               bias: Optional[torch.Tensor] = None, per_head: int = 0, rate: float = 0.0, in_act: Optional[str] = None) -> torch.Tensor:
+    """The second product of a low-rank projection: float32 [n, N] = f(g(x[:, col0: col0 + r]) @ weight_t), ``x`` float32
     rows (the first product's sums), ``weight_t`` float32 [r, N].  f: ``plain``; ``sigmoid``; ``decay``:
-    exp(-exp(a_log[c // per_head]) * softplus(sum + bias[c]))."""
+    exp(-exp(a_log[c // per_head]) * softplus(sum + bias[c])); ``rate_sigmoid``: exp(-rate * sigmoid(sum + bias[c])).
+    g: the identity, or tanh with ``in_act`` ``"tanh"``."""
+    _need(in_act in (None, "tanh"), f"lowrank_up: input function {in_act!r} unknown")
     if _backend is not None:
+        if mode == "rate_sigmoid" or in_act is not None:
+            return _backend.lowrank_up(x, col0, weight_t, mode, a_log, bias, per_head, rate, in_act)
         return _backend.lowrank_up(x, col0, weight_t, mode, a_log, bias, per_head)
     _dev_ok(x, weight_t, a_log, bias)
     _need(mode in LOWRANK_MODES, f"lowrank_up: mode {mode!r} unknown")
@@ -1301,9 +1324,11 @@ def lowrank_up(x: torch.Tensor, col0: int, weight_t: torch.Tensor, mode: str = "
     if mode == "decay":
         _need(a_log is not None and bias is not None and per_head > 0 and n_out % per_head == 0 and a_log.dtype == torch.float32
               and bias.dtype == torch.float32 and a_log.numel() == n_out // per_head and bias.numel() == n_out, "lowrank_up: bad decay constants")
+    if mode == "rate_sigmoid":
+        _need(bias is not None and bias.dtype == torch.float32 and bias.numel() == n_out, "lowrank_up: bad decay biases")
     out = torch.empty((x.shape[0], n_out), dtype=torch.float32, device=x.device)
     _call("tp_lowrank_up", _ptr(x), x.shape[1], int(col0), r, _ptr(weight_t), _ptr(out), x.shape[0], n_out, LOWRANK_MODES[mode],
-          _ptr(a_log), _ptr(bias), int(per_head), _stream())
+          _ptr(a_log), _ptr(bias), int(per_head), 1 if in_act == "tanh" else 0, ctypes.c_float(rate), _stream())
     return out
 
 
@@ -1338,19 +1363,31 @@ def delta_scan(qkv: torch.Tensor, decay: torch.Tensor, proj: torch.Tensor, beta_
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: Optional[torch.Tensor], eps: float, scale: float, heads: int,
-                   out: torch.Tensor, out_col0: int) -> None:
+                   out: torch.Tensor, out_col0: int, gate_rows: Optional[torch.Tensor] = None, gate_col0: int = 0) -> None:
     """out[:, out_col0 + h * vdim + d] = o[:, h, d] / sqrt(mean_d o^2 + eps) * weight[d] * gate[:, h * vdim + d] * scale:
-    ``o`` float32 [n, heads * vdim], ``weight`` float32 [vdim] shared by the heads, ``gate`` float32 like ``o`` or None."""
+    ``o`` float32 [n, heads * vdim]; ``weight`` float32 [vdim] shared by the heads, or [heads * vdim], every head its own;
+    ``gate`` float32 like ``o`` or None.  ``gate_rows`` (float32 rows [n, wider], instead of ``gate``): the gate is the
+    sigmoid of their columns gate_col0 .. gate_col0 + heads * vdim."""
     if _backend is not None:
+        if gate_rows is not None:
+            return _backend.head_norm_gate(o, weight, gate, eps, scale, heads, out, out_col0, gate_rows, gate_col0)
         return _backend.head_norm_gate(o, weight, gate, eps, scale, heads, out, out_col0)
-    _dev_ok(o, weight, gate, out)
+    _dev_ok(o, weight, gate, out, gate_rows)
     _need(o.dtype == torch.float32 and o.dim() == 2 and o.shape[1] % heads == 0, "head_norm_gate: o must be float32 [n, heads * vdim]")
     n, vdim = o.shape[0], o.shape[1] // heads
-    _need(weight.dtype == torch.float32 and weight.numel() == vdim, "head_norm_gate: weight must be float32 [vdim]")
+    _need(weight.dtype == torch.float32 and weight.numel() in (vdim, heads * vdim), "head_norm_gate: weight must be float32 [vdim] or [heads * vdim]")
+    # (one head: a weight of [vdim] is both)
+    per_head = int(weight.numel() == heads * vdim and heads > 1)
+    _need(gate is None or gate_rows is None, "head_norm_gate: one gate")
     _need(gate is None or (gate.dtype == torch.float32 and tuple(gate.shape) == tuple(o.shape)), "head_norm_gate: gate must match o")
     _need(out.dim() == 2 and out.shape[0] == n and 0 <= out_col0 and out_col0 + o.shape[1] <= out.shape[1], "head_norm_gate: output rows too short")
-    _call("tp_head_norm_gate", _ptr(o), _ptr(weight), _ptr(gate), ctypes.c_float(eps), ctypes.c_float(scale), _ptr(out), _dt(out),
-          out.shape[1], int(out_col0), n, int(heads), vdim, _stream())
+    gate_ptr, gate_stride, raw = _ptr(gate), o.shape[1], 0
+    if gate_rows is not None:
+        _need(gate_rows.dtype == torch.float32 and gate_rows.dim() == 2 and gate_rows.shape[0] == n and 0 <= gate_col0
+              and gate_col0 + o.shape[1] <= gate_rows.shape[1], "head_norm_gate: bad gate rows")
+        gate_ptr, gate_stride, raw = ctypes.c_void_p(gate_rows.data_ptr() + 4 * int(gate_col0)), gate_rows.shape[1], 1
+    _call("tp_head_norm_gate", _ptr(o), _ptr(weight), gate_ptr, ctypes.c_float(eps), ctypes.c_float(scale), _ptr(out), _dt(out),
+          out.shape[1], int(out_col0), n, int(heads), vdim, per_head, ctypes.c_size_t(gate_stride), raw, _stream())
 
 
 def moe_plan(ids: torch.Tensor, experts: int):
@@ -1410,4 +1447,104 @@ def moe_spread(a: torch.Tensor, dense: torch.Tensor, experts: int) -> torch.Tens
     n, ff = a.shape[0], a.shape[1] // experts
     out = torch.empty((experts, n, ff), dtype=a.dtype, device=a.device)
     _call("tp_moe_spread", _ptr(a), _dt(a), _ptr(dense), _ptr(out), n, int(experts), ff, _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------------
+# Operations of layers with one norm for both sublayers, inputs convolved over time, a generalized delta rule, an
+# attention over keys and values expanded from a latent, and a vector added to the stream between layers.
+
+def rmsnorm_cols(x: torch.Tensor, col0: int, width: int, weight: torch.Tensor, eps: float, out_dtype: torch.dtype, groups: int = 1) -> torch.Tensor:
+    """The RMS norm (in ``groups`` equal parts) of columns col0 .. col0 + width of float32 rows [n, wider], times
+    ``weight`` [width] -> out_dtype [n, width]."""
+    if _backend is not None:
+        return _backend.rmsnorm_cols(x, col0, width, weight, eps, out_dtype, groups)
+    _dev_ok(x, weight)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and 0 <= col0 and col0 + width <= x.shape[1], "rmsnorm_cols: bad rows")
+    _need(weight.dtype == torch.float32 and weight.numel() == width and groups > 0 and width % groups == 0, "rmsnorm_cols: bad weight or groups")
+    out = torch.empty((x.shape[0], width), dtype=out_dtype, device=x.device)
+    _call("tp_group_rmsnorm", _ptr(x), ctypes.c_size_t(x.shape[1]), int(col0), _ptr(weight), _ptr(None), _ptr(out), _dtcode(out_dtype),
+          x.shape[0], int(width), int(groups), ctypes.c_float(eps), _stream())
+    return out
+
+
+def residual_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, state_off: int, cu_seqlens: torch.Tensor,
+                  token_req: torch.Tensor, state_slots: torch.Tensor, num_requests: int, out_dtype: torch.dtype):
+    """What sublayers read of rows ``x`` (float32 [n, width]): for each of the ``weight`` [subs, taps, width] (tap-major,
+    the last tap the current token's) x + conv(x) over each request's run of tokens, as ``out_dtype``; a list of
+    ``subs`` tensors [n, width].  ``state`` float32 [slots, row]: from element ``state_off`` on a request's carried
+    rows [taps - 1, width] (oldest first), read for the first tokens of a run and replaced by the run's last rows."""
+    if _backend is not None:
+        return _backend.residual_conv(x, weight, state, state_off, cu_seqlens, token_req, state_slots, num_requests, out_dtype)
+    _dev_ok(x, weight, state, cu_seqlens, token_req, state_slots)
+    _need(x.dtype == torch.float32 and x.dim() == 2, "residual_conv: rows must be float32 [n, width]")
+    n, width = x.shape
+    _need(weight.dtype == torch.float32 and weight.dim() == 3 and weight.shape[2] == width, "residual_conv: weight must be float32 [subs, taps, width]")
+    subs, taps = weight.shape[0], weight.shape[1]
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state_off >= 0 and state.shape[1] >= state_off + (taps - 1) * width,
+          "residual_conv: state rows too short")
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    _i32(token_req, n, "token_req") if n else None
+    out = torch.empty((subs, n, width), dtype=out_dtype, device=x.device)
+    _call("tp_residual_conv", _ptr(x), _ptr(weight), _ptr(state), ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off),
+          _ptr(cu_seqlens), _ptr(token_req), _ptr(state_slots), _ptr(out), _dtcode(out_dtype), n, int(num_requests), width, taps, subs,
+          _stream())
+    return [out[i] for i in range(subs)]
+
+
+def add_row(h: torch.Tensor, table: torch.Tensor, row: int) -> None:
+    """h[t] += table[row] for every row t, in place (float32)."""
+    if _backend is not None:
+        return _backend.add_row(h, table, row)
+    _dev_ok(h, table)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and table.dtype == torch.float32 and table.dim() == 2 and table.shape[1] == h.shape[1]
+          and 0 <= row < table.shape[0], "add_row: h float32 [n, width], table float32 [rows, width]")
+    _call("tp_add_row", _ptr(h), ctypes.c_void_p(table.data_ptr() + 4 * int(row) * table.shape[1]), h.shape[0], h.shape[1], _stream())
+
+
+def general_delta_scan(proj: torch.Tensor, col0: int, decay: torch.Tensor, a_bias: torch.Tensor, state: torch.Tensor, state_off: int,
+                       cu_seqlens: torch.Tensor, state_slots: torch.Tensor, num_requests: int, heads: int, dim: int,
+                       unit_eps: float) -> torch.Tensor:
+    """The generalized delta rule per head over each request's run.  ``proj`` float32 rows hold, from column ``col0``
+    on, r | k | v | a_raw, each [heads * dim]; a = sigmoid(a_raw + a_bias); ``decay`` float32 [n, heads * dim].  With the
+    unit key u = k / sqrt(sum k^2 + unit_eps) and S [dim, dim] per head (kept at ``state[slot, state_off:]`` column by
+    column):  S <- diag(decay) S - (a u) (u^T S) + k v^T (both terms read the old S);  o = S^T r.
+    Returns o float32 [n, heads * dim]; the state is left as the run leaves it."""
+    if _backend is not None:
+        return _backend.general_delta_scan(proj, col0, decay, a_bias, state, state_off, cu_seqlens, state_slots, num_requests, heads, dim, unit_eps)
+    _dev_ok(proj, decay, a_bias, state, cu_seqlens, state_slots)
+    n, hd = proj.shape[0], heads * dim
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and 0 <= col0 and col0 + 4 * hd <= proj.shape[1], "general_delta_scan: bad r | k | v | a rows")
+    _need(decay.dtype == torch.float32 and tuple(decay.shape) == (n, hd), "general_delta_scan: decay must be float32 [n, heads * dim]")
+    _need(a_bias.dtype == torch.float32 and a_bias.numel() == hd, "general_delta_scan: a_bias must be float32 [heads * dim]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state_off >= 0 and state.shape[1] >= state_off + hd * dim,
+          "general_delta_scan: state rows too short")
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    y = torch.empty((n, hd), dtype=torch.float32, device=proj.device)
+    scratch = torch.empty((max(1, n * 2 * hd + n * heads * 2),), dtype=torch.float32, device=proj.device)
+    _call("tp_gdelta_scan", _ptr(proj), proj.shape[1], int(col0), _ptr(decay), _ptr(a_bias), _ptr(state), ctypes.c_size_t(state.shape[1]),
+          ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(y), _ptr(scratch), n, int(num_requests), int(heads),
+          int(dim), ctypes.c_float(unit_eps), _stream())
+    return y
+
+
+def latent_rows(proj: torch.Tensor, q_col0: int, rot_col0: int, up: torch.Tensor, heads: int, dim: int, rot: int, vdim: int) -> torch.Tensor:
+    """The rows q | k | v that ``rope_kv_write`` takes, for an attention whose keys and values are expanded from a
+    latent: q [heads, rot + dim] is columns q_col0 .. of ``proj`` (float32 rows) as they stand; head h's key is the
+    shared part proj[:, rot_col0 : rot_col0 + rot] followed by up[:, h * dim : (h + 1) * dim]; its value
+    up[:, heads * dim + h * vdim : ...].  ``up`` float32 [n, >= heads * (dim + vdim)].  Returns float32
+    [n, 2 * heads * (rot + dim) + heads * vdim]."""
+    if _backend is not None:
+        return _backend.latent_rows(proj, q_col0, rot_col0, up, heads, dim, rot, vdim)
+    _dev_ok(proj, up)
+    n = proj.shape[0]
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and up.dtype == torch.float32 and up.dim() == 2 and up.shape[0] == n,
+          "latent_rows: float32 rows")
+    _need(0 <= q_col0 and q_col0 + heads * (rot + dim) <= proj.shape[1] and 0 <= rot_col0 and rot_col0 + rot <= proj.shape[1]
+          and up.shape[1] >= heads * (dim + vdim), "latent_rows: rows too short")
+    out = torch.empty((n, 2 * heads * (rot + dim) + heads * vdim), dtype=torch.float32, device=proj.device)
+    _call("tp_latent_rows", _ptr(proj), ctypes.c_size_t(proj.shape[1]), int(q_col0), int(rot_col0), _ptr(up), ctypes.c_size_t(up.shape[1]),
+          _ptr(out), n, int(heads), int(dim), int(rot), int(vdim), _stream())
     return out

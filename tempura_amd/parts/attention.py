@@ -341,3 +341,93 @@ class ConvAttention(BranchMixer):
 
 
 register_part("mixer", "conv_attention", ConvAttention)
+
+
+class LatentAttention(BranchMixer):
+    """Softmax attention whose keys and values are expanded from one compressed vector per token.  With H =
+    ``num_heads``, per head D = ``head_dim`` unrotated and R = ``rotary_dim`` rotated query/key elements, values of
+    ``value_dim`` and a latent of L = ``latent_dim``: q = W_q x, per head [D unrotated | R rotated]; W_down x has L + R
+    rows: the first L, RMS-normed (``norm_eps``) with a weight, are the latent c, the last R (not normed) are ONE rotated
+    key part shared by all heads.  Head h's unrotated key is W_uk[h] c, its value W_uv[h] c; the score is
+    (q_plain . k_plain + q_rot . k_rot) * ``scale``.  The position part rotates neighbouring pairs (2i, 2i + 1) of the R
+    rotated elements of q and of the shared key part.  ``window``, ``gate`` (sigmoid(W_g x) on the concatenated heads) as
+    for ``conv_attention``.
+
+    The cache holds expanded keys and values per head: keys [rotated | unrotated] of R + D, values of ``value_dim``.
+    Every model of this kind here runs under a sliding window, which bounds what a request holds, and a decode step
+    then needs no products with the expansion weights for the keys it reads.  At load the rows of W_q are brought into
+    the cache's order per head, [rotated | unrotated]; q and k are ordered alike, so no score changes.
+
+    The columns of its input product are [q | down | gate]; it keeps no per-request state."""
+    preferred_portion_align = 8      # (the value cache is transposed: see ``PagedAttention``)
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.num_heads = int(p["num_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.rotary_dim = int(p["rotary_dim"])
+        self.value_dim = int(p["value_dim"])
+        self.latent_dim = int(p["latent_dim"])
+        self.scale = float(p["scale"])
+        self.window = p.get("window")
+        self.norm_eps = float(p["norm_eps"])
+        self.gate = bool(p.get("gate", False))
+        self.position = build_part("position", p["position"], hidden_size, dtype, device)
+        rot = self.position.rotary()
+        if (rot[1] if rot is not None else 0) != self.rotary_dim:
+            raise ValueError("latent_attention: the position part must rotate exactly the rotated elements")
+        self.key_dim = self.head_dim + self.rotary_dim
+        self.q_dim = self.num_heads * self.key_dim
+        self.down_dim = self.latent_dim + self.rotary_dim
+        self.inner = self.num_heads * self.value_dim
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        p, w = spec.params, spec.weights
+        H, D, R, Dv, L = (int(p[k]) for k in ("num_heads", "head_dim", "rotary_dim", "value_dim", "latent_dim"))
+        out = {w["q"]: WeightInfo((H * (D + R), hidden_size)), w["down"]: WeightInfo((L + R, hidden_size)),
+               w["latent_norm"]: WeightInfo((L,), "ones"), w["up_k"]: WeightInfo((H * D, L)), w["up_v"]: WeightInfo((H * Dv, L)),
+               w["o"]: WeightInfo((hidden_size, H * Dv))}
+        if p.get("gate", False):
+            out[w["gate"]] = WeightInfo((H * Dv, hidden_size))
+        out.update(part_class("position", p["position"].kind).expected_weights(p["position"], hidden_size))
+        return out
+
+    def cache_spec(self):
+        kind = "window" if self.window is not None else "full"
+        if self.value_dim == self.key_dim:
+            return CacheSpec(kind, self.num_heads, self.key_dim, self.window)
+        return SizedValueCacheSpec(kind, self.num_heads, self.key_dim, self.window, self.value_dim)
+
+    def load_branch(self, get):
+        from .base import pad_rows
+        w = self.spec.weights
+        H, D, R = self.num_heads, self.head_dim, self.rotary_dim
+        q = get(w["q"])
+        q = torch.cat([q.view(H, D + R, -1)[:, D:], q.view(H, D + R, -1)[:, :D]], dim=1).reshape(q.shape)      # per head [rotated | unrotated]
+        rows = [q, get(w["down"])]
+        if self.gate:
+            rows.append(get(w["gate"]))
+        self.latent_norm_w = self._to_device(get(w["latent_norm"]), torch.float32)
+        self.w_up = ops.tile_weight(pad_rows(torch.cat([self._to_device(get(w["up_k"])), self._to_device(get(w["up_v"]))], dim=0), 16))
+        self.position.load_weights(get)
+        return torch.cat([self._to_device(t) for t in rows], dim=0).contiguous(), self._to_device(get(w["o"]))
+
+    def run(self, proj, col0, ctx, cache, out, out_col0, scale):
+        if not cache.writes:
+            raise ValueError("latent_attention: a call that reads another call's cache is not supported")
+        H = self.num_heads
+        c = ops.rmsnorm_cols(proj, col0 + self.q_dim, self.latent_dim, self.latent_norm_w, self.norm_eps, self.dtype)
+        up = ops.linear(c, self.w_up, torch.float32)
+        rows = ops.latent_rows(proj, col0, col0 + self.q_dim + self.latent_dim, up, H, self.head_dim, self.rotary_dim, self.value_dim)
+        inv_freq, rotary_dim, factor = self.position.rotary()
+        table = self.position.table(ctx) if hasattr(self.position, "table") else None
+        q = ops.rope_kv_write(rows, ctx.positions, ctx.slot_mapping[cache.group], inv_freq, rotary_dim, factor, H, H, self.key_dim,
+                              cache.k, cache.v, self.dtype, table, value_dim=self.value_dim)
+        a = ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+                                ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len, ctx.num_single)
+        ops.sigmoid_gate(a, proj if self.gate else None, col0 + self.q_dim + self.down_dim, scale, out, out_col0)
+
+
+register_part("mixer", "latent_attention", LatentAttention)

@@ -161,7 +161,7 @@ class HyperBlock(ArrangedBlock):
 
     @staticmethod
     def _opening(norm, link):
-        if hasattr(norm, "weight") and hasattr(norm, "eps") and type(norm).__name__ == "RMSNorm":
+        if hasattr(norm, "weight") and hasattr(norm, "eps") and type(norm).__name__ == "RMSNorm" and getattr(norm, "groups", 1) == 1:
             return StreamOpening(None if link is None else link.in_coef, norm.weight, norm.eps)
         return None
 
@@ -230,7 +230,7 @@ class SandwichBlock(ArrangedBlock):
         if len({self.ffn is None, self.ffn_norm is None, self.ffn_post_norm is None}) != 1:
             raise ValueError("block 'sandwich': a feed-forward and its two norms come together")
         for post in (self.mixer_post_norm, self.ffn_post_norm):
-            if post is not None and type(post).__name__ != "RMSNorm":
+            if post is not None and (type(post).__name__ != "RMSNorm" or getattr(post, "groups", 1) != 1):
                 raise ValueError("block 'sandwich': the norm behind a sublayer must be an RMS norm")
         self.hidden_size = hidden_size
         self.dtype = dtype
@@ -238,7 +238,7 @@ class SandwichBlock(ArrangedBlock):
     @staticmethod
     def _rms(norm):
         """(weight, eps) of an RMS norm that the closing kernel can apply, else None."""
-        if type(norm).__name__ == "RMSNorm":
+        if type(norm).__name__ == "RMSNorm" and getattr(norm, "groups", 1) == 1:
             return norm.weight, norm.eps
         return None
 
@@ -278,3 +278,52 @@ class SandwichBlock(ArrangedBlock):
 
 
 register_part("block", "sandwich", SandwichBlock)
+
+
+class SharedNormBlock(ArrangedBlock):
+    """ONE norm whose output both sublayers read, their outputs entering the stream together:
+    n = norm(h); h += mixer(in_0(n)) + ffn(in_1(n)).  ``inputs`` (optional, category ``input``) says what each sublayer
+    reads of n (``residual_conv``: n plus a short convolution of n over time, one weight per sublayer); without it both
+    read n itself.  A layer may have no feed-forward.
+
+    The layer's state row holds the input part's carried rows first and the mixer's state behind them, so the mixer is
+    one that takes an offset into its row (a ``BranchMixer``) or keeps no state."""
+    ROLES = {"norm": "norm", "inputs": "input", "mixer": "mixer", "ffn": "ffn"}
+    OPTIONAL = frozenset({"inputs", "ffn"})
+
+    def __init__(self, layer_spec, hidden_size, dtype, device):
+        super().__init__(layer_spec, hidden_size, dtype, device)
+        self.dtype = dtype
+        self.front = self.inputs.state_floats() if self.inputs is not None else 0
+        if self.front:
+            if self.mixer.state_spec() is not None and not hasattr(self.mixer, "state_floats"):
+                raise ValueError(f"block 'shared_norm': mixer {self.mixer.spec.kind!r} cannot share a state row (no state offset)")
+            if hasattr(self.mixer, "state_floats"):
+                self.mixer.state_off = self.front
+        if self.inputs is not None and len(self.inputs.names) != (1 if self.ffn is None else 2):
+            raise ValueError("block 'shared_norm': the input part needs one weight per sublayer")
+
+    def cache_owner(self):
+        return self
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def state_spec(self):
+        from .base import StateSpec
+        if not self.front:
+            return self.mixer.state_spec()
+        behind = self.mixer.state_floats() if hasattr(self.mixer, "state_floats") else 0
+        return StateSpec((self.front + behind,), torch.float32)
+
+    def forward(self, h, ctx, cache) -> None:
+        if self.inputs is not None:
+            xs = self.inputs.forward(self.norm.forward(h, out_dtype=torch.float32), ctx, cache)
+        else:
+            xs = [self.norm.forward(h)] * 2
+        self.mixer.forward(xs[0], ctx, cache, h)
+        if self.ffn is not None:
+            self.ffn.forward(xs[1], ctx, h)
+
+
+register_part("block", "shared_norm", SharedNormBlock)

@@ -97,3 +97,64 @@ class GatedDeltaMixer(BranchMixer):
 
 
 register_part("mixer", "gated_delta", GatedDeltaMixer)
+
+
+class GeneralDeltaMixer(BranchMixer):
+    """A generalized delta-rule mixer.  With H = ``num_heads`` heads of D = ``head_dim``: r, k, v = W_r x, W_k x, W_v x
+    [H, D]; a decay per head and key channel w = exp(-``decay_rate`` * sigmoid(W_w2 tanh(W_w1 x) + w0)); a removal rate
+    per head and key channel a = sigmoid(W_a x + a_bias).  With the unit key u = k / sqrt(sum k^2 + ``unit_eps``), per
+    head and with S [D, D] starting at zero:
+
+        S <- diag(w) S - (a u) (u^T S) + k v^T        (both terms read the old S)        o = S^T r
+
+    o is divided by its root mean square per head (``norm_eps``), the concatenated heads times a weight [H D], times
+    sigmoid(W_g x), then projected back.  Everything between the projections is float32 whatever the compute dtype.
+
+    The columns of its input product are [r | k | v | a | gate | w1]; the rank of the decay's low-rank projection is the
+    checkpoint's own.  Per request it keeps the state in one float32 row (a head's matrix column by column: [H, D, D])."""
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.num_heads = int(p["num_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.norm_eps = float(p["norm_eps"])
+        self.unit_eps = float(p.get("unit_eps", 1e-6))
+        self.decay_rate = float(p["decay_rate"])
+        self.inner = self.num_heads * self.head_dim
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        p, w = spec.params, spec.weights
+        n = int(p["num_heads"]) * int(p["head_dim"])
+        rank = p.get("decay_rank")
+        out = {w[name]: WeightInfo((n, hidden_size)) for name in ("r", "k", "v", "gate", "a")}
+        out.update({w["a_bias"]: WeightInfo((n,)), w["w1"]: WeightInfo((rank, hidden_size)), w["w2"]: WeightInfo((n, rank)),
+                    w["w0"]: WeightInfo((n,)), w["norm"]: WeightInfo((n,), "ones"), w["o"]: WeightInfo((hidden_size, n))})
+        return out
+
+    def state_floats(self) -> int:
+        return self.num_heads * self.head_dim * self.head_dim
+
+    def load_branch(self, get):
+        w = self.spec.weights
+        f32 = lambda name: self._to_device(get(w[name]), torch.float32)
+        w1, w2 = get(w["w1"]), f32("w2")
+        if w2.shape[1] != w1.shape[0]:
+            raise ValueError("general_delta: the two halves of the decay's projection disagree on its rank")
+        self.w2_t = w2.t().contiguous()      # [rank, columns]: lanes read neighbours
+        self.a_bias, self.w0, self.norm_w = f32("a_bias"), f32("w0"), f32("norm")
+        rows = [get(w["r"]), get(w["k"]), get(w["v"]), get(w["a"]), get(w["gate"]), w1]
+        self.gate_col = 4 * self.inner
+        self.w1_col = 5 * self.inner
+        return torch.cat([self._to_device(t) for t in rows], dim=0).contiguous(), self._to_device(get(w["o"]))
+
+    def run(self, proj, col0, ctx, cache, out, out_col0, scale):
+        decay = ops.lowrank_up(proj, col0 + self.w1_col, self.w2_t, "rate_sigmoid", bias=self.w0, rate=self.decay_rate, in_act="tanh")
+        o = ops.general_delta_scan(proj, col0, decay, self.a_bias, cache.state, self.state_off, ctx.cu_seqlens, ctx.state_slots,
+                                   ctx.num_requests, self.num_heads, self.head_dim, self.unit_eps)
+        ops.head_norm_gate(o, self.norm_w, None, self.norm_eps, scale, self.num_heads, out, out_col0, gate_rows=proj,
+                           gate_col0=col0 + self.gate_col)
+
+
+register_part("mixer", "general_delta", GeneralDeltaMixer)

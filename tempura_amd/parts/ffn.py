@@ -152,7 +152,12 @@ class RoutedExperts(FeedForward):
     has (the one wait of the layer), every expert with rows is one pair of products over its rows, and a token's
     sum adds its experts' rows in the order of its choice.  Either way a row's result does not depend on what else
     is in the batch; the two ways differ in rounding only.  Tensor roles: ``router``,
-    ``correction``, and ``gate`` / ``up`` / ``down`` as name patterns with ``{}`` for the expert's number."""
+    ``correction``, and ``gate`` / ``up`` / ``down`` as name patterns with ``{}`` for the expert's number.
+
+    Parameters of the router beyond that: ``score`` (``"softmax"`` or ``"sigmoid"``: s = sigmoid(logit), each expert by
+    itself); a spec without a ``correction`` tensor has none; ``group_best`` (default 1): a group is ranked by the sum
+    of that many of its largest choice scores; ``normalize``: the weights are the chosen s over their sum (plus
+    ``sum_eps``); ``scale`` multiplies the weights."""
     graph_safe = True
     returns_output = True
 
@@ -170,6 +175,16 @@ class RoutedExperts(FeedForward):
         if self.groups > 1 and (self.experts % self.groups != 0 or not 0 < self.keep <= self.groups
                                 or self.keep * (self.experts // self.groups) < self.top):
             raise ValueError("moe: groups must divide the experts and the kept groups must hold at least top experts")
+        self.score = str(p.get("score", "softmax"))
+        if self.score not in ops.ROUTE_SCORES:
+            raise ValueError(f"moe: score {self.score!r} unknown (known: {sorted(ops.ROUTE_SCORES)})")
+        self.group_best = int(p.get("group_best", 1))
+        self.normalize = bool(p.get("normalize", False))
+        self.sum_eps = float(p.get("sum_eps", 0.0))
+        self.weight_scale = float(p.get("scale", 1.0))
+        if self.group_best < 1:
+            raise ValueError("moe: group_best must be at least 1")
+        self.plain_router = (self.score, self.group_best, self.normalize, self.weight_scale) == ("softmax", 1, False, 1.0)
         self.w_router = self.correction = None
         self.w13, self.w2 = [], []
 
@@ -177,7 +192,9 @@ class RoutedExperts(FeedForward):
     def expected_weights(cls, spec, hidden_size):
         p, w = spec.params, spec.weights
         i, e = p["intermediate_size"], p["experts"]
-        out = {w["router"]: WeightInfo((e, hidden_size)), w["correction"]: WeightInfo((e,))}
+        out = {w["router"]: WeightInfo((e, hidden_size))}
+        if "correction" in w:
+            out[w["correction"]] = WeightInfo((e,))
         for n in range(e):
             out[w["gate"].format(n)] = WeightInfo((i, hidden_size))
             out[w["up"].format(n)] = WeightInfo((i, hidden_size))
@@ -188,7 +205,7 @@ class RoutedExperts(FeedForward):
         from .base import pad_rows
         w = self.spec.weights
         self.w_router = ops.tile_weight(pad_rows(self._to_device(get(w["router"])), 16))
-        self.correction = self._to_device(get(w["correction"]), torch.float32)
+        self.correction = self._to_device(get(w["correction"]), torch.float32) if "correction" in w else None
         self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
         stack, self.w2 = [], []
         for n in range(self.experts):
@@ -209,7 +226,12 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x, ctx, residual=None):
         logits = ops.linear(x, self.w_router, torch.float32)
-        dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
+        if self.plain_router and self.correction is not None:
+            dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
+        else:
+            dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep, score=self.score,
+                                                group_best=self.group_best, normalize=self.normalize, sum_eps=self.sum_eps,
+                                                scale=self.weight_scale)
         if getattr(ctx, "max_q_len", 1) <= 1:
             if self.fused:
                 a = ops.linear_swiglu(x, self.w13_all)

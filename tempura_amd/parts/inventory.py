@@ -14,6 +14,9 @@ def expected_weights(spec: ModelSpec) -> Dict[str, WeightInfo]:
         spec.embedding, spec.hidden_size, spec.vocab_size))
     for ls in spec.layers:
         out.update(part_class("block", ls.block).expected_weights(ls, spec.hidden_size))
+    for call in spec.order:
+        if call.before is not None:
+            out.update(part_class("stream", call.before.kind).expected_weights(call.before, spec.hidden_size))
     out.update(part_class("norm", spec.final_norm.kind).expected_weights(spec.final_norm, spec.hidden_size))
     out.update(part_class("lm_head", spec.lm_head.kind).expected_weights(
         spec.lm_head, spec.hidden_size, spec.vocab_size))

@@ -1,5 +1,8 @@
 """RMSNorm: ``y = x / sqrt(mean(x^2) + eps) * (w + weight_offset)``.
 
+``groups`` (default 1): the row is split into that many equal consecutive parts and each is divided by its own root
+mean square; the weight spans the whole row.
+
 ``weight_offset`` (default 0) serves checkpoints that store the weight around zero: with 1.0 the stored tensor is
 the deviation from one.  The offset is added once, in float32, when the weight is loaded.
 ``scale`` (default 1) multiplies the result: a norm behind a sublayer whose output enters the residual stream
@@ -25,6 +28,9 @@ class RMSNorm(Norm):
         self.eps = float(spec.params["eps"])
         self.weight_offset = float(spec.params.get("weight_offset", 0.0))
         self.scale = float(spec.params.get("scale", 1.0))
+        self.groups = int(spec.params.get("groups", 1) or 1)
+        if self.groups < 1 or hidden_size % self.groups != 0:
+            raise ValueError(f"rmsnorm: groups ({self.groups}) must divide the row ({hidden_size})")
         self.weight = None
 
     @classmethod
@@ -41,13 +47,16 @@ class RMSNorm(Norm):
         if self.scale != 1.0:
             self.weight = (self.weight.double() * self.scale).to(torch.float32)
 
-    def forward(self, h, rows=None):
-        return ops.rmsnorm(h, self.weight, self.eps, self.dtype, rows)
+    def forward(self, h, rows=None, out_dtype=None):
+        """``out_dtype``: another type than the compute dtype (float32 rows for a part that goes on in float32)."""
+        if self.groups > 1:
+            return ops.rmsnorm(h, self.weight, self.eps, out_dtype or self.dtype, rows, groups=self.groups)
+        return ops.rmsnorm(h, self.weight, self.eps, out_dtype or self.dtype, rows)
 
     def deferred(self, m):
         """(weight, eps) when the two products around this norm can carry it for ``m`` rows (the one
         before prepares, the one after applies the scale), else None."""
-        if ops.split_norm_ok(m, self.hidden_size, self.dtype):
+        if self.groups == 1 and ops.split_norm_ok(m, self.hidden_size, self.dtype):
             return self.weight, self.eps
         return None
 

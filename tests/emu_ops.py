@@ -121,12 +121,63 @@ class EmuOps:
         v = v / torch.sqrt((v * v).mean(dim=-1, keepdim=True) + eps)
         return (v.reshape(n, inner) * weight.double()).to(out_dtype)
 
-    def rmsnorm(self, h, weight, eps, out_dtype, rows=None):
+    def rmsnorm(self, h, weight, eps, out_dtype, rows=None, groups=1):
         x = h.double()
         if rows is not None:
             x = x[rows.long()]
-        y = x * (1.0 / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)) * weight.double()
+        p = x.reshape(x.shape[0], groups, x.shape[1] // groups)
+        y = (p * (1.0 / torch.sqrt((p * p).mean(dim=-1, keepdim=True) + eps))).reshape(x.shape) * weight.double()
         return y.to(out_dtype)
+
+    def rmsnorm_cols(self, x, col0, width, weight, eps, out_dtype, groups=1):
+        return self.rmsnorm(x[:, col0: col0 + width], weight, eps, out_dtype, None, groups)
+
+    def residual_conv(self, x, weight, state, state_off, cu_seqlens, token_req, state_slots, num_requests, out_dtype):
+        subs, taps, width = weight.shape
+        out = torch.zeros(subs, x.shape[0], width, dtype=torch.float64)
+        cu = cu_seqlens.tolist()
+        lo, hi = state_off, state_off + (taps - 1) * width
+        for r in range(num_requests):
+            a, e = cu[r], cu[r + 1]
+            if e <= a:
+                continue
+            slot = int(state_slots[r])
+            seq = torch.cat([state[slot, lo:hi].double().reshape(taps - 1, width), x[a:e].double()], dim=0)
+            for t in range(e - a):
+                for sub in range(subs):
+                    out[sub, a + t] = seq[t + taps - 1] + (seq[t: t + taps] * weight[sub].double()).sum(0)
+            state[slot, lo:hi] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
+        return [out[sub].to(out_dtype) for sub in range(subs)]
+
+    def add_row(self, h, table, row):
+        h.add_(table[row])
+
+    def general_delta_scan(self, proj, col0, decay, a_bias, state, state_off, cu_seqlens, state_slots, num_requests, heads, dim, unit_eps):
+        n, hd = proj.shape[0], heads * dim
+        x = proj.double()
+        r, k, v, ar = (x[:, col0 + i * hd: col0 + (i + 1) * hd].reshape(n, heads, dim) for i in range(4))
+        a = torch.sigmoid(ar + a_bias.double().reshape(heads, dim))
+        w = decay.double().reshape(n, heads, dim)
+        y = torch.zeros(n, heads, dim, dtype=torch.float64)
+        cu = cu_seqlens.tolist()
+        for q in range(num_requests):
+            slot = int(state_slots[q])
+            # (kept column by column: [heads, value, key])
+            S = state[slot, state_off: state_off + hd * dim].double().reshape(heads, dim, dim).transpose(1, 2).clone()
+            for t in range(cu[q], cu[q + 1]):
+                u = k[t] / torch.sqrt((k[t] * k[t]).sum(-1, keepdim=True) + unit_eps)
+                seen = torch.einsum("hd,hdv->hv", u, S)
+                S = w[t][:, :, None] * S - (a[t] * u)[:, :, None] * seen[:, None, :] + k[t][:, :, None] * v[t][:, None, :]
+                y[t] = torch.einsum("hdv,hd->hv", S, r[t])
+            state[slot, state_off: state_off + hd * dim] = S.transpose(1, 2).reshape(-1).to(torch.float32)
+        return y.reshape(n, hd).to(torch.float32)
+
+    def latent_rows(self, proj, q_col0, rot_col0, up, heads, dim, rot, vdim):
+        n, key = proj.shape[0], rot + dim
+        q = proj[:, q_col0: q_col0 + heads * key]
+        shared = proj[:, rot_col0: rot_col0 + rot][:, None, :].expand(n, heads, rot)
+        k = torch.cat([shared, up[:, : heads * dim].reshape(n, heads, dim)], dim=2).reshape(n, heads * key)
+        return torch.cat([q, k, up[:, heads * dim: heads * (dim + vdim)]], dim=1).to(torch.float32).contiguous()
 
     def split_norm_ok(self, m, width, dtype):
         return dtype == torch.bfloat16 and 0 < m <= 128 and width % 32 == 0
@@ -270,9 +321,12 @@ class EmuOps:
             v = z * torch.sigmoid(z)
         return v.to(out_dtype)
 
-    def moe_route(self, logits, correction, experts, top, groups, keep):
+    def moe_route(self, logits, correction, experts, top, groups, keep, score="softmax", group_best=1, normalize=False, sum_eps=0.0,
+                  scale=1.0):
         n = logits.shape[0]
-        s = torch.softmax(logits.double()[:, :experts], dim=-1)
+        s = torch.softmax(logits.double()[:, :experts], dim=-1) if score == "softmax" else torch.sigmoid(logits.double()[:, :experts])
+        if correction is None:
+            correction = torch.zeros(experts)
         dense = torch.zeros(n, experts, dtype=torch.float32)
         ids = torch.zeros(n, top, dtype=torch.int32)
         wts = torch.zeros(n, top, dtype=torch.float32)
@@ -280,14 +334,15 @@ class EmuOps:
             ch = (s[t] + correction.double()).tolist()
             if groups > 1:
                 per = experts // groups
-                score = [max(ch[g * per: (g + 1) * per]) for g in range(groups)]
+                score = [sum(sorted(ch[g * per: (g + 1) * per], reverse=True)[:group_best]) for g in range(groups)]
                 kept = sorted(range(groups), key=lambda g: (-score[g], g))[:keep]
                 ch = [c if e // per in kept else float("-inf") for e, c in enumerate(ch)]
             order = [e for e in sorted(range(experts), key=lambda e: (-ch[e], e)) if ch[e] != float("-inf")][:top]
+            factor = scale / (sum(float(s[t, e]) for e in order) + sum_eps) if normalize else scale
             for i, e in enumerate(order):
-                dense[t, e] = s[t, e]
+                dense[t, e] = s[t, e] * factor
                 ids[t, i] = e
-                wts[t, i] = s[t, e]
+                wts[t, i] = s[t, e] * factor
         return dense, ids, wts
 
     def moe_plan(self, ids, experts):
@@ -320,9 +375,12 @@ class EmuOps:
         n, ff = a.shape[0], a.shape[1] // experts
         return (a.double().reshape(n, experts, ff) * dense.double()[:, :, None]).permute(1, 0, 2).contiguous().to(a.dtype)
 
-    def lowrank_up(self, x, col0, weight_t, mode="plain", a_log=None, bias=None, per_head=0):
+    def lowrank_up(self, x, col0, weight_t, mode="plain", a_log=None, bias=None, per_head=0, rate=0.0, in_act=None):
         r = weight_t.shape[0]
-        v = x.double()[:, col0: col0 + r] @ weight_t.double()
+        xin = x.double()[:, col0: col0 + r]
+        v = (torch.tanh(xin) if in_act == "tanh" else xin) @ weight_t.double()
+        if mode == "rate_sigmoid":
+            v = torch.exp(-rate * torch.sigmoid(v + bias.double()))
         if mode == "sigmoid":
             v = torch.sigmoid(v)
         elif mode == "decay":
@@ -359,12 +417,15 @@ class EmuOps:
             state[slot, state_off: state_off + size] = S.transpose(1, 2).reshape(-1).to(torch.float32)
         return y.reshape(n, heads * vdim).to(torch.float32)
 
-    def head_norm_gate(self, o, weight, gate, eps, scale, heads, out, out_col0):
+    def head_norm_gate(self, o, weight, gate, eps, scale, heads, out, out_col0, gate_rows=None, gate_col0=0):
         n, vdim = o.shape[0], o.shape[1] // heads
         x = o.double().reshape(n, heads, vdim)
-        x = (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight.double()).reshape(n, heads * vdim)
+        w = weight.double().reshape(-1, vdim)      # [1, vdim] shared or [heads, vdim]
+        x = (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w).reshape(n, heads * vdim)
         if gate is not None:
             x = x * gate.double()
+        if gate_rows is not None:
+            x = x * torch.sigmoid(gate_rows.double()[:, gate_col0: gate_col0 + heads * vdim])
         out[:, out_col0: out_col0 + heads * vdim] = (x * scale).to(out.dtype)
 
     def swiglu(self, gu, out_dtype):
