@@ -376,8 +376,10 @@ class GolavikConfig:
         for i, l in enumerate(self.layers):
             p = f"l{i}"
             taps = [f"{p}.canon1"] + ([f"{p}.canon2"] if l.mlp is not None else [])
+            # (a layer without a feed-forward has no use for the second convolution; a checkpoint may hold it all the same)
+            names = {"taps": taps} if l.mlp is not None else {"taps": taps, "unused": [f"{p}.canon2"]}
             parts = {"norm": norm(f"{p}.norm1"), "mixer": l.mixer.part(f"{p}.mix", self.norm_eps),
-                     "inputs": PartSpec("residual_conv", {"taps": self.canon_taps}, {"taps": taps})}
+                     "inputs": PartSpec("residual_conv", {"taps": self.canon_taps}, names)}
             if l.mlp is not None:
                 parts["ffn"] = l.mlp.part(f"{p}.mlp")
             layers.append(LayerSpec("shared_norm", parts))

@@ -1481,13 +1481,14 @@ def residual_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, st
     n, width = x.shape
     _need(weight.dtype == torch.float32 and weight.dim() == 3 and weight.shape[2] == width, "residual_conv: weight must be float32 [subs, taps, width]")
     subs, taps = weight.shape[0], weight.shape[1]
-    _need(state.dtype == torch.float32 and state.dim() == 2 and state_off >= 0 and state.shape[1] >= state_off + (taps - 1) * width,
-          "residual_conv: state rows too short")
+    # (one tap carries nothing: a layer whose parts keep no state then has no state tensor)
+    _need((state is None and taps == 1) or (state is not None and state.dtype == torch.float32 and state.dim() == 2 and state_off >= 0
+                                            and state.shape[1] >= state_off + (taps - 1) * width), "residual_conv: state rows too short")
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
     _i32(token_req, n, "token_req") if n else None
     out = torch.empty((subs, n, width), dtype=out_dtype, device=x.device)
-    _call("tp_residual_conv", _ptr(x), _ptr(weight), _ptr(state), ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off),
+    _call("tp_residual_conv", _ptr(x), _ptr(weight), _ptr(state), ctypes.c_size_t(0 if state is None else state.shape[1]), ctypes.c_size_t(state_off),
           _ptr(cu_seqlens), _ptr(token_req), _ptr(state_slots), _ptr(out), _dtcode(out_dtype), n, int(num_requests), width, taps, subs,
           _stream())
     return [out[i] for i in range(subs)]

@@ -4,7 +4,8 @@
 its own ([hidden, taps], no bias; conv(n)_t = sum_j w[:, j] n_(t - taps + 1 + j), zeros before a request's start).
 The sublayers convolve the SAME rows, so a request carries the last ``taps - 1`` normed rows once, whatever the number
 of sublayers: ``state_floats()`` float32 values of its state row, from ``state_off`` on.  Sums are float32; the results
-come in the compute dtype, one tensor per sublayer (tensor role ``taps``: a list of names, one per sublayer).
+come in the compute dtype, one tensor per sublayer (tensor role ``taps``: a list of names, one per sublayer; role
+``unused``, optional: names of weights a checkpoint may hold for sublayers the layer does not have, which are ignored).
 """
 from __future__ import annotations
 
@@ -29,7 +30,10 @@ class ResidualConv(Part):
 
     @classmethod
     def expected_weights(cls, spec, hidden_size):
-        return {name: WeightInfo((hidden_size, int(spec.params["taps"]))) for name in spec.weights["taps"]}
+        shape = (hidden_size, int(spec.params["taps"]))
+        out = {name: WeightInfo(shape) for name in spec.weights["taps"]}
+        out.update({name: WeightInfo(shape, "skip", optional=True) for name in spec.weights.get("unused", [])})
+        return out
 
     def state_floats(self) -> int:
         return (self.taps - 1) * self.hidden_size

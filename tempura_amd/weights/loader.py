@@ -200,7 +200,7 @@ def load_into(model, model_dir: str, verify: Optional[bool] = None) -> None:
     # but the user should know that it is not what runs
     ignored = sorted(n for n, info in expected.items() if info.init == "skip" and n in have)
     if ignored:
-        warnings.warn(f"checkpoint in {model_dir} holds {', '.join(ignored)}, but the configuration ties that tensor to "
-                      f"another (tie_word_embeddings): the stored tensor is ignored", stacklevel=2)
+        warnings.warn(f"checkpoint in {model_dir} holds {', '.join(ignored)}, which the configuration does not use (a tied "
+                      f"output head, a sublayer the layer does not have): the stored tensor is ignored", stacklevel=2)
     model.load_weights(get)
     ckpt.close()

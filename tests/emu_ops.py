@@ -142,11 +142,13 @@ class EmuOps:
             if e <= a:
                 continue
             slot = int(state_slots[r])
-            seq = torch.cat([state[slot, lo:hi].double().reshape(taps - 1, width), x[a:e].double()], dim=0)
+            carried = state[slot, lo:hi].double().reshape(taps - 1, width) if taps > 1 else torch.zeros(0, width, dtype=torch.float64)
+            seq = torch.cat([carried, x[a:e].double()], dim=0)
             for t in range(e - a):
                 for sub in range(subs):
                     out[sub, a + t] = seq[t + taps - 1] + (seq[t: t + taps] * weight[sub].double()).sum(0)
-            state[slot, lo:hi] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
+            if taps > 1:
+                state[slot, lo:hi] = seq[seq.shape[0] - (taps - 1):].reshape(-1).to(torch.float32)
         return [out[sub].to(out_dtype) for sub in range(subs)]
 
     def add_row(self, h, table, row):
