@@ -69,11 +69,16 @@ CASES: Dict[str, dict] = {
 }
 
 
-def config_json(name: str) -> dict:
-    """The case as config.json would hold it (without the tests' private keys)."""
+def config_json(name: str, every_expert: bool = False) -> dict:
+    """The case as config.json would hold it (without the tests' private keys).  ``every_expert``: each token uses
+    all experts, without groups, so that no choice is there for a rounding to flip (for runs in bfloat16; the scores
+    still weigh the experts)."""
     cfg = json.loads(json.dumps(CASES[name]))
     for layer in cfg["layers"]:
         layer["mixer"].pop("_ranks", None)
+        if every_expert and layer["mlp"] is not None:
+            layer["mlp"]["router"]["top"] = layer["mlp"]["router"]["experts"]
+            layer["mlp"]["router"].pop("groups", None)
     return cfg
 
 
