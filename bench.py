@@ -58,7 +58,7 @@ def parse_args():
     ap.add_argument("--mixed-chunk", type=int, default=512)
     ap.add_argument("--mixed-temperature", type=float, default=0.0, help="0: greedy; above: seeded sampling with top-k 50")
     ap.add_argument("--decode-target-blocks", type=int, default=None, help="tuning: blocks the split decode attention aims at")
-    ap.add_argument("--design", default=None, choices=["mifutar", "bomotar"],
+    ap.add_argument("--design", default=None, choices=["mifutar", "bomotar", "golavik"],
                     help="instead of the headline: prefill and decode throughput of this design at layer sizes of real models, "
                          "beside Llama layers of equal size, with the time of every kernel entry point")
     ap.add_argument("--design-sizes", default="2048,4096", help="model widths of --design (comma separated)")
@@ -79,9 +79,14 @@ def design_bench(args) -> int:
     Llama layer's heads (values as wide as keys, four taps, YaRN rotation) beside a delta rule of width / 128 heads
     of 128 x 128 (low-rank projections of rank 64), and feed-forwards that alternate between a dense one and eight
     experts of a quarter of its width, two a token out of two of four groups; it stands beside the Mifutar model and
-    the Llama layers (no window there).  Prints one JSON line."""
+    the Llama layers (no window there).  A Golavik model here has layers of a channel delta rule (width / 128 heads of
+    128 x 128, ranks 64), a general delta rule (width / 64 heads of 64), a latent attention of the Llama layer's heads
+    (three quarters of a head unrotated, a quarter rotated, values as wide as the whole key, a latent of 512, window
+    1,024) and a channel delta rule again, each with eight experts of a quarter of the dense width, two a token out of
+    two of four groups, a norm in eight parts and four taps on the inputs; it stands beside the Bomotar model and the
+    Llama layers.  Prints one JSON line."""
     import torch
-    from tempura_amd.config import BomotarConfig, LlamaConfig, MifutarConfig
+    from tempura_amd.config import BomotarConfig, GolavikConfig, LlamaConfig, MifutarConfig
     from tempura_amd.engine import Engine
     from tempura_amd.engine.loading import random_model
     from tempura_amd.engine.runner import StepEntry
@@ -116,6 +121,18 @@ def design_bench(args) -> int:
         return BomotarConfig.from_dict({"architecture": "Bomotar", "vocab": vocab, "width": width, "residual_mult": 0.8,
                                         "norm": {"eps": 1e-6}, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
                                         "layers": ls, "max_positions": 8192})
+
+    def golavik_config(width, ff, heads, dim, kv, layers):
+        channel = {"heads": width // 128, "kv_heads": width // 128, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+        general = {"heads": width // 64, "dim": 64, "decay_rank": 64}
+        latent = {"heads": heads, "dim": 3 * dim // 4, "rot_dim": dim // 4, "vdim": dim, "kv_rank": 512, "scale": dim ** -0.5,
+                  "mask": {"size": window},
+                  "rot": {"dims": dim // 4, "base": 1000000.0, "scaling": {"factor": 4.0, "original": 2048, "fast": 16.0, "slow": 2.0}}}
+        moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+        kinds = [("channel_delta", channel), ("general_delta", general), ("latent_attention", latent), ("channel_delta", channel)]
+        ls = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": moe} for i in range(layers)]
+        return GolavikConfig.from_dict({"architecture": "Golavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 8},
+                                        "canon": {"taps": 4}, "layers": ls, "max_positions": 8192})
 
     def llama_config(width, ff, heads, dim, kv, layers):
         return LlamaConfig(width, ff, layers, heads, kv, dim, vocab, 8192, 1e-5, 500000.0, None, False,
@@ -173,6 +190,9 @@ def design_bench(args) -> int:
                   ("llama", llama_config(width, ff, heads, dim, kv, args.design_layers))]
         if design == "bomotar":
             models.insert(0, ("bomotar", bomotar_config(width, ff, heads, dim, kv, args.design_layers)))
+        if design == "golavik":
+            models = [("golavik", golavik_config(width, ff, heads, dim, kv, args.design_layers)),
+                      ("bomotar", bomotar_config(width, ff, heads, dim, kv, args.design_layers)), models[1]]
         chosen = [m for m in args.design_models.split(",") if m]
         for name, cfg in [m for m in models if not chosen or m[0] in chosen]:
             say(f"{name} width {width}: building")
@@ -187,7 +207,8 @@ def design_bench(args) -> int:
                       "n_gpus": 1, "higher_is_better": True, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic", "vs_baseline": None,
                       "config": {"design": {"mifutar": "Mifutar beside Llama layers of equal size",
-                                            "bomotar": "Bomotar beside Mifutar and Llama layers of equal size"}[design],
+                                            "bomotar": "Bomotar beside Mifutar and Llama layers of equal size",
+                                            "golavik": "Golavik beside Bomotar and Llama layers of equal size"}[design],
                                  "layers": args.design_layers, "prompt": T, "decode_batch": batch,
                                  "window": window if design == "mifutar" else None}, "points": points}))
     return 0
