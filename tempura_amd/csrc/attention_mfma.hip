@@ -92,6 +92,10 @@ struct AttnArgs {
   // float32, entry min(query position - key position, bias_len - 1); nullptr: none
   const float* dist_bias;
   int bias_len;
+  // the kernel whose blocks share keys and values through LDS: how many heads of a key group a block's four waves
+  // take (4, 2 or 1); with 2 or 1 the waves left over take further query tiles of the same heads, so that a model
+  // with as many key heads as heads has no idle waves
+  int heads_per_block;
 };
 #define PART_STRIDE(D) ((D) + 4)
 
@@ -419,7 +423,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_
 }
 
 // ---- prefill, keys and values through LDS ---------------------------------------------------
-// The four waves of a block (four heads of one kv group) need the same keys and values.  Here a
+// The four waves of a block (four heads of one kv group; with one or two heads a group, 4 or 2 query tiles of each
+// head: AttnArgs::heads_per_block) need the same keys and values.  Here a
 // step's 32 keys and values are copied once per block into LDS by the direct global-to-LDS load,
 // NS - 1 steps ahead of their use (a ring of NS stages, three or four; one barrier per step), and every wave reads
 // its operand fragments from there: a quarter of the global load instructions, and none of their
@@ -471,11 +476,14 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
   const int q_start = a.cu_seqlens[r];
   const int q_len = a.cu_seqlens[r + 1] - q_start;
   if (q_len <= 0 || (skip_single && q_len == 1)) return;
-  const int nqb = (q_len + 16 * NQ - 1) / (16 * NQ);
+  // a block's waves: heads_per_block heads of one key group times 4 / heads_per_block query tiles (of 16 NQ rows)
+  const int hpb = a.heads_per_block;
+  const int rows_b = 16 * NQ * (4 / hpb);
+  const int nqb = (q_len + rows_b - 1) / rows_b;
   if (bx >= nqb) return;
   const int group = a.n_heads / a.n_kv;
   const int kvh = by % a.n_kv;
-  const int hin = (by / a.n_kv) * 4 + wave;
+  const int hin = (by / a.n_kv) * hpb + (wave & (hpb - 1));
   const bool active = hin < group;     // a wave without a head still loads and waits with the others
   const int head = kvh * group + min(hin, group - 1);
   const int ctx = a.context_lens[r];
@@ -483,7 +491,8 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
   const int* table = a.block_tables + (size_t)r * a.table_width;
   const int ps = a.page_size;
 
-  const int q0 = (nqb - 1 - bx) * 16 * NQ;
+  const int qb0 = (nqb - 1 - bx) * rows_b;          // the block's first query row
+  const int q0 = qb0 + (wave / hpb) * 16 * NQ;      // this wave's (past the portion's end: it computes the last row again and writes nothing)
   bf16x8_t qf[NQ][D / 32];
   int qpos[NQ];
   float m[NQ], l[NQ];
@@ -500,9 +509,11 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
 #pragma unroll
     for (int dt = 0; dt < D / 16; ++dt) o[nq][dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   }
-  const int last_pos = pos0 + min(q0 + 16 * NQ, q_len) - 1;
+  // the block walks the keys that any of its rows sees; a wave masks what its own rows do not see
+  const int last_pos = pos0 + min(qb0 + rows_b, q_len) - 1;
+  const int last_mine = pos0 + min(q0 + 16 * NQ, q_len) - 1;   // the last query of this wave
   int first = 0;
-  if (a.window > 0) first = max(0, pos0 + q0 - a.window + 1) & ~31;
+  if (a.window > 0) first = max(0, pos0 + qb0 - a.window + 1) & ~31;
   int nsteps = (last_pos - first) / 32 + 1;
   const int my_parts = portion_parts(nsteps, a.portion_splits, a.portion_min_steps);
   if (part >= my_parts) return;
@@ -511,7 +522,7 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     first += s_begin * 32;
     nsteps = s_end - s_begin;
   }
-  const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this block
+  const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this wave
   if constexpr (BIAS) {
     for (int i = lane; i < a.bias_len; i += 64) bias_lds[wave * ATTN_BIAS_LDS + i] = a.dist_bias[(size_t)head * a.bias_len + i];
     __syncthreads();
@@ -672,7 +683,7 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     bool moved[NQ];
     u32x4_t vv[D / 16];
     const int j0 = first + s * 32;
-    const bool plain_step = j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_pos - a.window + 1);
+    const bool plain_step = j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_mine - a.window + 1);
 #define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<(dt >> 1) * 2048 + (dt & 1) * 256>(base + vaddr)
 #define ATTN_BODY(NEXT, MASK)                                                                          \
   {                                                                                                    \
@@ -1017,6 +1028,21 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
       if (g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
+        if (group <= 2) {
+          // one or two heads a key group: a block takes them all and 4 / group query tiles of each (its four waves
+          // share the keys and values of 64 or 128 rows instead of three or two of them idling)
+          a.heads_per_block = group;
+          const int tiles = 4 / group;
+          const long wide2 = (long)((n_tokens - num_single + 32 * tiles - 1) / (32 * tiles) + (n_req - num_single - 1)) * a.n_kv;
+          const bool two_w = g_attn_tune == 2 || (g_attn_tune != 3 && wide2 >= 768);
+          const int rows_w = (two_w ? 32 : 16) * tiles;
+          const dim3 wgrid((max_q_len + rows_w - 1) / rows_w, a.n_kv, n_req);
+          if (two_w)
+            hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), wgrid, dim3(256), 0, s, a, skip);
+          else
+            hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 1, 3, 3>), wgrid, dim3(256), 0, s, a, skip);
+          return 0;
+        }
         if (two)
           hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), grid, dim3(256), 0, s, a, skip);
         else
@@ -1069,6 +1095,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
   a.token_req = token_req;
   a.dist_bias = dist_bias;
   a.bias_len = bias_len;
+  a.heads_per_block = 4;
   if (dist_bias != nullptr && bias_len <= 0) return -1;
   a.scale_log2 = scale * 1.4426950408889634f;
   switch (head_dim) {

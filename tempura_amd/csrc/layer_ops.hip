@@ -672,6 +672,52 @@ __global__ void residual_conv_kernel(const float* __restrict__ x, const float* _
   }
 }
 
+// the same, four neighbouring channels a thread (width a multiple of four, at most four sublayers): 16-byte loads of
+// the rows and the weights; the request's carried rows are read element by element (their place in the state row
+// need not be aligned).  Every channel's sum is formed in the order of the kernel above: the same bits.
+#define RCONV_MAX_SUBS 4
+template <typename TO>
+__global__ void residual_conv4_kernel(const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ state,
+                                      size_t state_stride, size_t state_off, const int* __restrict__ cu_seqlens,
+                                      const int* __restrict__ token_req, const int* __restrict__ state_slots, TO* __restrict__ out,
+                                      size_t out_stride_sub, int width, int taps, int subs, int channel_blocks) {
+  const int t = blockIdx.x / channel_blocks;
+  const int c = ((blockIdx.x % channel_blocks) * blockDim.x + threadIdx.x) * 4;
+  if (c >= width) return;
+  const int r = token_req[t];
+  const int start = cu_seqlens[r];
+  const int i = t - start;
+  const float* st = state + (size_t)state_slots[r] * state_stride + state_off;
+  const float4 cur = *(const float4*)(x + (size_t)t * width + c);
+  float4 acc[RCONV_MAX_SUBS];
+#pragma unroll
+  for (int sub = 0; sub < RCONV_MAX_SUBS; ++sub) acc[sub] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = 0; k < taps; ++k) {
+    const int src = i - (taps - 1 - k);
+    float4 v;
+    if (src >= 0) {
+      v = *(const float4*)(x + (size_t)(start + src) * width + c);
+    } else {
+      const float* p = st + (size_t)(taps - 1 + src) * width + c;
+      v = make_float4(p[0], p[1], p[2], p[3]);
+    }
+#pragma unroll
+    for (int sub = 0; sub < RCONV_MAX_SUBS; ++sub)
+      if (sub < subs) {
+        const float4 wv = *(const float4*)(w + ((size_t)sub * taps + k) * width + c);
+        acc[sub].x = fmaf(wv.x, v.x, acc[sub].x);
+        acc[sub].y = fmaf(wv.y, v.y, acc[sub].y);
+        acc[sub].z = fmaf(wv.z, v.z, acc[sub].z);
+        acc[sub].w = fmaf(wv.w, v.w, acc[sub].w);
+      }
+  }
+#pragma unroll
+  for (int sub = 0; sub < RCONV_MAX_SUBS; ++sub)
+    if (sub < subs)
+      from_float4(out + (size_t)sub * out_stride_sub + (size_t)t * width + c, cur.x + acc[sub].x, cur.y + acc[sub].y,
+                  cur.z + acc[sub].z, cur.w + acc[sub].w);
+}
+
 __global__ void residual_conv_state_kernel(const float* __restrict__ x, float* __restrict__ state, size_t state_stride,
                                            size_t state_off, const int* __restrict__ cu_seqlens,
                                            const int* __restrict__ state_slots, int width, int taps) {
@@ -698,7 +744,18 @@ extern "C" int tp_residual_conv(const float* x, const float* w, float* state, si
   const int cb = (width + threads - 1) / threads;
   TP_REQUIRE(cb <= 65535 && (long)n * cb < 0x7fffffffL, "residual_conv: too many channels or tokens");
   const size_t sub_stride = (size_t)n * width;
-  if (out_dt == TP_F32)
+  TP_REQUIRE(out_dt == TP_F32 || out_dt == TP_BF16, "residual_conv: unknown dtype %d", out_dt);
+  if (width % 4 == 0 && subs <= RCONV_MAX_SUBS && (((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) & 15) == 0) {
+    const int quads = width / 4;
+    const int qthreads = quads >= 256 ? 256 : 64;
+    const int qb = (quads + qthreads - 1) / qthreads;
+    if (out_dt == TP_F32)
+      hipLaunchKernelGGL(residual_conv4_kernel<float>, dim3((unsigned)((long)n * qb)), dim3(qthreads), 0, s, x, w, state, state_stride,
+                         state_off, cu_seqlens, token_req, state_slots, (float*)out, sub_stride, width, taps, subs, qb);
+    else
+      hipLaunchKernelGGL(residual_conv4_kernel<bf16_t>, dim3((unsigned)((long)n * qb)), dim3(qthreads), 0, s, x, w, state, state_stride,
+                         state_off, cu_seqlens, token_req, state_slots, (bf16_t*)out, sub_stride, width, taps, subs, qb);
+  } else if (out_dt == TP_F32)
     hipLaunchKernelGGL(residual_conv_kernel<float>, dim3((unsigned)((long)n * cb)), dim3(threads), 0, s, x, w, state, state_stride,
                        state_off, cu_seqlens, token_req, state_slots, (float*)out, sub_stride, width, taps, subs, cb);
   else if (out_dt == TP_BF16)

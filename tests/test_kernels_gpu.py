@@ -655,6 +655,22 @@ def test_attention_mfma(heads, kv, d, page):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("heads,kv,d,page", [(4, 4, 64, 16), (3, 3, 128, 32), (6, 3, 128, 16), (2, 1, 32, 64), (8, 8, 32, 16)])
+def test_attention_mfma_with_one_or_two_heads_a_key_group(heads, kv, d, page):
+    """Key groups of one or two heads: the waves of a block that have no head of their own take further query tiles of
+    the same heads, so a block spans 64 to 128 query rows and walks every key one of them sees.  Portions that end
+    inside a block, start in the middle of a cached prefix, are shorter than a block, and windows shorter and longer
+    than a block's rows; 16 and 32 rows a wave give the same bits."""
+    bf = torch.bfloat16
+    _attention_case(bf, heads, kv, d, page, [200, 75, 1, 17], [200, 139, 90, 17], 0, seed=31)
+    _attention_case(bf, heads, kv, d, page, [130, 1, 66], [257, 300, 66], 40, seed=32)
+    _attention_case(bf, heads, kv, d, page, [97, 64], [400, 64], 150, seed=33)
+    _attention_case(bf, heads, kv, d, page, [3, 129], [35, 129], 1, seed=34)
+    for q_lens, ctx_lens, window in (([170, 33, 1], [170, 97, 40], 0), ([145, 100], [300, 100], 50), ([260], [260], 96)):
+        a, b = (_attention_case(bf, heads, kv, d, page, q_lens, ctx_lens, window, seed=35, tune=t) for t in (2, 3))
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("heads,kv,d,page", [(8, 2, 128, 16), (6, 3, 64, 32), (5, 1, 32, 64)])
 def test_attention_portions_with_split_keys(heads, kv, d, page):
     """Few query blocks under a long context: the keys of a portion are split over blocks and the parts combined.
