@@ -31,6 +31,10 @@ def _window_of(spec: CacheSpec) -> int:
     return int(spec.window) if spec.window is not None else 0
 
 
+def _kept_of(spec: CacheSpec) -> int:
+    return int(getattr(spec, "keep_first", 0) or 0)
+
+
 _RULES: Dict[str, VisibilityRule] = {
     # every key stays visible: pages are held until the request ends
     "full": VisibilityRule(0, lambda s: (), lambda s, total, step: total),
@@ -40,6 +44,9 @@ _RULES: Dict[str, VisibilityRule] = {
     # the keys of the query's own aligned chunk of `window` positions
     "chunk": VisibilityRule(2, lambda s: (_window_of(s),),
                             lambda s, total, step: min(total, _window_of(s) + step) if _window_of(s) > 0 else total),
+    # the last `window` keys and, for good, the request's first `keep_first` keys (their pages are never given back)
+    "window_keep_first": VisibilityRule(3, lambda s: (_window_of(s), _kept_of(s)),
+                                        lambda s, total, step: min(total, _window_of(s) + step + _kept_of(s)) if _window_of(s) > 0 else total),
 }
 
 

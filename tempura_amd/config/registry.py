@@ -15,6 +15,7 @@ from .llama import ConfigError, LlamaConfig
 from .mifutar import MifutarConfig
 from .bomotar import BomotarConfig
 from .golavik import GolavikConfig
+from .zemarax import ZemaraxConfig
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -76,3 +77,4 @@ register_architecture("llama", LlamaConfig)
 register_architecture("Mifutar", MifutarConfig)
 register_architecture("Bomotar", BomotarConfig)
 register_architecture("Golavik", GolavikConfig)
+register_architecture("Zemarax", ZemaraxConfig)

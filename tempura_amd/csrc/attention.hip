@@ -11,6 +11,11 @@
 // context_lens[r] - q_len_r + (t - cu_seqlens[r]) and it sees keys lo..pos with
 // lo = max(0, pos - window + 1) when window > 0, else 0.
 //
+// Kept first keys: with keep_first > 0 a windowed query also sees keys 0..keep_first-1 (those of them that lie
+// before lo; they are visited first, so the order of keys stays ascending).
+// Sink: with sink [heads] float32 the softmax's denominator holds one more term, exp(sink[h]), that has no key and
+// no value; it is added once, after the last key, whatever the scale.
+//
 // Optional bias by distance: dist_bias [heads, bias_len] float32 is added to the scaled score of query position
 // pos and key j as dist_bias[h, min(pos - j, bias_len - 1)] (the scale does not multiply it).
 #include <math.h>
@@ -25,7 +30,7 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_seqlens,
     const int* __restrict__ context_lens, const int* __restrict__ token_req, T* __restrict__ out, int n_heads,
     int n_kv, int head_dim, int page_size, float scale, int window, const float* __restrict__ dist_bias, int bias_len,
-    int value_dim) {
+    int value_dim, int keep_first, const float* __restrict__ sink) {
   extern __shared__ float qs[];  // the query row, float32
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = token_req[t];
@@ -44,9 +49,13 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
 #pragma unroll
   for (int i = 0; i < ATT_MAX_ACC; ++i) acc[i] = 0.f;
 
-  for (int j0 = lo; j0 <= pos; j0 += TP_WAVE) {
+  // two runs of keys: the kept first ones that the window has left behind, then the window (or everything)
+  const int kept_end = (keep_first > 0 && lo > 0) ? min(keep_first, lo) : 0;
+  for (int seg = kept_end > 0 ? 0 : 1; seg < 2; ++seg) {
+  const int seg_lo = seg == 0 ? 0 : lo, seg_hi = seg == 0 ? kept_end - 1 : pos;
+  for (int j0 = seg_lo; j0 <= seg_hi; j0 += TP_WAVE) {
     const int j = j0 + lane;
-    const bool valid = j <= pos;
+    const bool valid = j <= seg_hi;
     int row = 0;   // cache row of this lane's key: (page * n_kv + kvh) * page_size + offset
     int vbase = 0; // its value column: values are stored [page, kv_head, head_dim, page_size]
     float s = -INFINITY;
@@ -67,7 +76,7 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
     m = m_new;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_ACC; ++i) acc[i] *= alpha;
-    const int n_valid = min(TP_WAVE, pos - j0 + 1);
+    const int n_valid = min(TP_WAVE, seg_hi - j0 + 1);
     for (int jj = 0; jj < n_valid; ++jj) {
       const float pj = __shfl(p, jj, TP_WAVE);
       const int vb = __shfl(vbase, jj, TP_WAVE);
@@ -78,6 +87,15 @@ __global__ __launch_bounds__(64) void paged_attention_kernel(
         if (d < value_dim) acc[i] = fmaf(pj, to_float(vr[(size_t)d * page_size]), acc[i]);
       }
     }
+  }
+  }
+  if (sink != nullptr) {
+    const float sk = sink[h];
+    const float m_new = fmaxf(m, sk);
+    const float alpha = expf(m - m_new);
+    l = l * alpha + expf(sk - m_new);
+#pragma unroll
+    for (int i = 0; i < ATT_MAX_ACC; ++i) acc[i] *= alpha;
   }
   const float inv = 1.0f / l;
   T* o = out + ((size_t)t * n_heads + h) * value_dim;
@@ -94,7 +112,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
                             int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
                             int portion_splits, int portion_min_steps, float* portion_scratch, const float* dist_bias,
-                            int bias_len, hipStream_t s);
+                            int bias_len, int keep_first, const float* sink, hipStream_t s);
 
 extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, const void* v_cache,
                                   const int* block_tables, int table_width, const int* cu_seqlens,
@@ -103,7 +121,7 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
                                   int window, int max_q_len, int max_ctx, int allow_fast, int num_single,
                                   int num_splits, float* scratch, int portion_splits, int portion_min_steps,
                                   float* portion_scratch, const float* dist_bias, int bias_len, int value_dim,
-                                  hipStream_t s) {
+                                  int keep_first, const float* sink, hipStream_t s) {
   // value_dim: the size of a value head (0: head_dim): v_cache is [page, kv_head, value_dim, page_size] and out
   // [n, heads * value_dim]; the matrix-core kernels take equal sizes only.
   if (value_dim <= 0) value_dim = head_dim;
@@ -117,6 +135,8 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   TP_REQUIRE(head_dim <= TP_WAVE * ATT_MAX_ACC && value_dim <= TP_WAVE * ATT_MAX_ACC, "paged_attention: head size %d / %d exceeds %d",
              head_dim, value_dim, TP_WAVE * ATT_MAX_ACC);
   TP_REQUIRE(window >= 0, "paged_attention: window must be >= 0");
+  TP_REQUIRE(keep_first >= 0, "paged_attention: keep_first must be >= 0");
+  if (window == 0) keep_first = 0;   // (without a window every key is seen anyway)
   TP_REQUIRE(n_heads <= 65535, "paged_attention: too many heads");
   if (n_tokens == 0) return 0;
   TP_REQUIRE(dist_bias == nullptr || bias_len > 0, "paged_attention: empty distance bias table");
@@ -124,7 +144,7 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
     const int rc = tp_paged_attention_fast(q, k_cache, v_cache, block_tables, table_width, cu_seqlens,
                                            context_lens, out, n_tokens, n_req, n_heads, n_kv, head_dim,
                                            page_size, scale, window, max_q_len, num_single, num_splits, scratch, token_req,
-                                           portion_splits, portion_min_steps, portion_scratch, dist_bias, bias_len, s);
+                                           portion_splits, portion_min_steps, portion_scratch, dist_bias, bias_len, keep_first, sink, s);
     if (rc >= 0) return rc;
   }
   const dim3 grid(n_tokens, n_heads);
@@ -132,11 +152,11 @@ extern "C" int tp_paged_attention(const void* q, int dt, const void* k_cache, co
   if (dt == TP_F32)
     hipLaunchKernelGGL(paged_attention_kernel<float>, grid, dim3(64), shmem, s, (const float*)q,
                        (const float*)k_cache, (const float*)v_cache, block_tables, table_width, cu_seqlens,
-                       context_lens, token_req, (float*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len, value_dim);
+                       context_lens, token_req, (float*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len, value_dim, keep_first, sink);
   else if (dt == TP_BF16)
     hipLaunchKernelGGL(paged_attention_kernel<bf16_t>, grid, dim3(64), shmem, s, (const bf16_t*)q,
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_seqlens,
-                       context_lens, token_req, (bf16_t*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len, value_dim);
+                       context_lens, token_req, (bf16_t*)out, n_heads, n_kv, head_dim, page_size, scale, window, dist_bias, bias_len, value_dim, keep_first, sink);
   else
     TP_REQUIRE(false, "paged_attention: unknown dtype %d", dt);
   TP_CHECK_LAUNCH("paged_attention");

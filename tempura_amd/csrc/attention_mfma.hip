@@ -1063,8 +1063,9 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int n_req, int n_heads, int n_kv, int head_dim, int page_size, float scale, int window,
                             int max_q_len, int num_single, int num_splits, float* scratch, const int* token_req,
                             int portion_splits, int portion_min_steps, float* portion_scratch, const float* dist_bias,
-                            int bias_len, hipStream_t s) {
+                            int bias_len, int keep_first, const float* sink, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
+  if (keep_first > 0 || sink != nullptr) return -1;   // (kept first keys and a sink run the general kernel)
   if (portion_min_steps < 1) return -1;
   if (portion_splits < 1 || portion_splits > 64 || (portion_splits > 1 && (portion_scratch == nullptr || token_req == nullptr))) return -1;
   if ((long)n_req * portion_splits > 65535) return -1;

@@ -92,8 +92,16 @@ typedef int (*FirstVisible)(int pos, const int* params);
 int rule_all(int, const int*) { return 0; }                                        // every key, always
 int rule_last_n(int pos, const int* p) { return p[0] > 0 ? std::max(0, pos - p[0] + 1) : 0; }   // a window of p[0] keys
 int rule_chunk(int pos, const int* p) { return p[0] > 0 ? pos / p[0] * p[0] : 0; }  // the query's own chunk of p[0] positions
-const FirstVisible RULES[] = {rule_all, rule_last_n, rule_chunk};
+// (code 3: a window of p[0] keys under which the first p[1] keys stay visible for good; the window part is rule_last_n,
+// the kept keys are what `kept_first` says)
+const FirstVisible RULES[] = {rule_all, rule_last_n, rule_chunk, rule_last_n};
 const int NUM_RULES = (int)(sizeof(RULES) / sizeof(RULES[0]));
+// A rule may also keep the first keys of a request visible whatever the position: their pages are never given back.
+// Per rule, the number of such keys (0: none).
+typedef int (*KeptFirst)(const int* params);
+int kept_none(const int*) { return 0; }
+int kept_p1(const int* p) { return p[0] > 0 ? std::max(0, p[1]) : 0; }
+const KeptFirst KEPT[] = {kept_none, kept_none, kept_none, kept_p1};
 
 struct Core {
   int page_size = 0, max_requests = 0;
@@ -105,6 +113,8 @@ struct Core {
   int n_groups() const { return (int)pools.size(); }
   // first logical page a query at position `start` can still see
   int first_needed(int g, int start) const { return RULES[rule[g]](start, &params[(size_t)g * RULE_PARAMS]) / page_size; }
+  // logical pages from 0 on that hold keys every query sees: held until the request ends
+  int kept_pages(int g) const { return (KEPT[rule[g]](&params[(size_t)g * RULE_PARAMS]) + page_size - 1) / page_size; }
   // pages group g must allocate so that the request can take n_new more tokens
   int pages_needed(const Request& r, int g, int n_new) const {
     const int end = r.num_tokens + n_new;
@@ -140,7 +150,7 @@ struct Core {
       const int keep_from = first_needed(g, r.num_tokens);
       std::vector<int>& table = r.tables[g];
       const int stop = std::min(keep_from, (int)table.size());
-      for (int lp = r.first_live[g]; lp < stop; ++lp)
+      for (int lp = std::max(r.first_live[g], kept_pages(g)); lp < stop; ++lp)
         if (table[lp] >= 0) {
           pools[g].release(table[lp]);
           table[lp] = -1;

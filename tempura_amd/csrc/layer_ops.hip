@@ -9,7 +9,7 @@
 __device__ inline float l_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
 
 // ---- embedding plus a row of a hashed bigram table --------------------------------------------
-// out[t] = table[token] + bigram[row], row = (previous * mul_prev + token * mul_cur) mod buckets, and row `buckets`
+// out[t] = table[token] * scale + bigram[row] (+ pos_table[position], a learned row per position), row = (previous * mul_prev + token * mul_cur) mod buckets, and row `buckets`
 // (the table's last) for the token at position 0.  The previous token is the one before it in the step's run, or,
 // for a run's first token, what the request's state row holds; a second kernel leaves each run's last token there.
 template <typename T>
@@ -17,18 +17,26 @@ __global__ void embed_bigram_kernel(const int* __restrict__ tokens, const int* _
                                     const int* __restrict__ token_req, const int* __restrict__ cu_seqlens,
                                     const int* __restrict__ state_slots, const int* __restrict__ prev_state,
                                     const T* __restrict__ table, const T* __restrict__ bigram, float* __restrict__ out,
-                                    int hidden, long long mul_prev, long long mul_cur, long long buckets) {
+                                    int hidden, long long mul_prev, long long mul_cur, long long buckets, float scale,
+                                    const T* __restrict__ pos_table) {
   const int t = blockIdx.x;
   const int tok = tokens[t];
   long long row = buckets;
-  if (positions[t] != 0) {
+  if (bigram != nullptr && positions[t] != 0) {
     const int r = token_req[t];
     const int prev = t > cu_seqlens[r] ? tokens[t - 1] : prev_state[state_slots[r]];
     row = ((long long)prev * mul_prev + (long long)tok * mul_cur) % buckets;
   }
   const T* a = table + (size_t)tok * hidden;
-  const T* b = bigram + (size_t)row * hidden;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) out[(size_t)t * hidden + c] = to_float(a[c]) + to_float(b[c]);
+  const T* b = bigram != nullptr ? bigram + (size_t)row * hidden : nullptr;
+  // (scale 1 and no position table: the sum of the two rows as it always was)
+  const T* p = pos_table != nullptr ? pos_table + (size_t)positions[t] * hidden : nullptr;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    float v = to_float(a[c]) * scale;
+    if (b != nullptr) v += to_float(b[c]);
+    if (p != nullptr) v += to_float(p[c]);
+    out[(size_t)t * hidden + c] = v;
+  }
 }
 
 __global__ void last_token_kernel(const int* __restrict__ tokens, const int* __restrict__ cu_seqlens,
@@ -42,19 +50,22 @@ __global__ void last_token_kernel(const int* __restrict__ tokens, const int* __r
 extern "C" int tp_embed_bigram(const int* tokens, const int* positions, const int* token_req, const int* cu_seqlens,
                                const int* state_slots, int* prev_state, const void* table, const void* bigram, int dt,
                                float* out, int n, int n_req, int hidden, long long mul_prev, long long mul_cur,
-                               long long buckets, hipStream_t s) {
-  TP_REQUIRE(n >= 0 && n_req >= 0 && hidden > 0 && buckets > 0 && mul_prev >= 0 && mul_cur >= 0, "embed_bigram: bad sizes");
+                               long long buckets, float scale, const void* pos_table, hipStream_t s) {
+  // (bigram may be missing: the token's row times scale, plus the position's row)
+  TP_REQUIRE(n >= 0 && n_req >= 0 && hidden > 0 && (bigram == nullptr || buckets > 0) && mul_prev >= 0 && mul_cur >= 0, "embed_bigram: bad sizes");
   if (n == 0) return 0;
   const int threads = hidden >= 256 ? 256 : 64;
   if (dt == TP_F32)
     hipLaunchKernelGGL(embed_bigram_kernel<float>, dim3(n), dim3(threads), 0, s, tokens, positions, token_req, cu_seqlens,
-                       state_slots, prev_state, (const float*)table, (const float*)bigram, out, hidden, mul_prev, mul_cur, buckets);
+                       state_slots, prev_state, (const float*)table, (const float*)bigram, out, hidden, mul_prev, mul_cur, buckets, scale,
+                       (const float*)pos_table);
   else if (dt == TP_BF16)
     hipLaunchKernelGGL(embed_bigram_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, tokens, positions, token_req, cu_seqlens,
-                       state_slots, prev_state, (const bf16_t*)table, (const bf16_t*)bigram, out, hidden, mul_prev, mul_cur, buckets);
+                       state_slots, prev_state, (const bf16_t*)table, (const bf16_t*)bigram, out, hidden, mul_prev, mul_cur, buckets, scale,
+                       (const bf16_t*)pos_table);
   else
     TP_REQUIRE(false, "embed_bigram: unknown dtype %d", dt);
-  if (n_req > 0)
+  if (n_req > 0 && bigram != nullptr)
     hipLaunchKernelGGL(last_token_kernel, dim3((n_req + 63) / 64), dim3(64), 0, s, tokens, cu_seqlens, state_slots, prev_state, n_req);
   TP_CHECK_LAUNCH("embed_bigram");
   return 0;
@@ -258,10 +269,44 @@ extern "C" int tp_norm_add(float* h, const float* y, const float* w, float eps, 
 }
 
 // ---- a plain activation -----------------------------------------------------------------------
-// kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))); kind 1: SiLU.
+// kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))); kind 1: SiLU; kind 2: the exact
+// GELU, 0.5 z (1 + erf(z / sqrt(2))).
 __device__ inline float act_f(float z, int kind) {
   if (kind == 0) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  if (kind == 2) return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
   return z * l_sigmoid(z);
+}
+
+// Rows of a wider float32 tensor: out[t, c] = act(in[t, col0 + c]) for c < width, times sigmoid(in[t, gate_col]) when
+// gate_col >= 0 (one gate a row: what a product behind it would be multiplied by, folded into its input).
+template <typename TO>
+__global__ void activation_rows_kernel(const float* __restrict__ in, size_t in_stride, int col0, int width, int gate_col,
+                                       TO* __restrict__ out, size_t total, int kind) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / width;
+  const int c = (int)(i % width);
+  const float* row = in + t * in_stride;
+  float v = act_f(row[col0 + c], kind);
+  if (gate_col >= 0) v *= l_sigmoid(row[gate_col]);
+  from_float(out + i, v);
+}
+
+extern "C" int tp_activation_rows(const float* in, size_t in_stride, int col0, int width, int gate_col, void* out, int out_dt, int n,
+                                  int kind, hipStream_t s) {
+  TP_REQUIRE(kind >= 0 && kind <= 2, "activation: unknown kind %d", kind);
+  TP_REQUIRE(n >= 0 && width > 0 && col0 >= 0 && (size_t)(col0 + width) <= in_stride && gate_col < (long)in_stride, "activation: bad rows");
+  const size_t total = (size_t)n * width;
+  if (total == 0) return 0;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (out_dt == TP_F32)
+    hipLaunchKernelGGL(activation_rows_kernel<float>, grid, dim3(256), 0, s, in, in_stride, col0, width, gate_col, (float*)out, total, kind);
+  else if (out_dt == TP_BF16)
+    hipLaunchKernelGGL(activation_rows_kernel<bf16_t>, grid, dim3(256), 0, s, in, in_stride, col0, width, gate_col, (bf16_t*)out, total, kind);
+  else
+    TP_REQUIRE(false, "activation: unknown dtype %d", out_dt);
+  TP_CHECK_LAUNCH("activation_rows");
+  return 0;
 }
 
 template <typename TI, typename TO>
@@ -281,7 +326,7 @@ __global__ void activation4_kernel(const float* __restrict__ in, TO* __restrict_
 }
 
 extern "C" int tp_activation(const void* in, int in_dt, void* out, int out_dt, size_t total, int kind, hipStream_t s) {
-  TP_REQUIRE(kind == 0 || kind == 1, "activation: unknown kind %d", kind);
+  TP_REQUIRE(kind >= 0 && kind <= 2, "activation: unknown kind %d", kind);
   if (total == 0) return 0;
   if (in_dt == TP_F32 && total % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0 && (out_dt == TP_F32 || out_dt == TP_BF16)) {
     const size_t total4 = total / 4;
@@ -337,7 +382,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
                                                         int groups, int keep, float* __restrict__ dense,
                                                         int* __restrict__ ids, float* __restrict__ weights, int n,
                                                         int score_kind, int group_best, int normalize, float sum_eps,
-                                                        float scale) {
+                                                        float scale, const float* __restrict__ logit_bias) {
   extern __shared__ float lds[];   // per wave: choice scores [experts], then group scores [groups]
   const int wave = threadIdx.x / TP_WAVE, lane = threadIdx.x % TP_WAVE;
   // (a wave past the last token works on the last token again and stores nothing: every wave reaches every barrier)
@@ -351,7 +396,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 #pragma unroll
   for (int k = 0; k < ROUTE_PER_LANE; ++k) {
     const int e = lane + k * TP_WAVE;
-    z[k] = e < experts ? logits[(size_t)t * logit_stride + e] : -INFINITY;
+    z[k] = e < experts ? logits[(size_t)t * logit_stride + e] + (logit_bias != nullptr ? logit_bias[e] : 0.f) : -INFINITY;
     mx = fmaxf(mx, z[k]);
     won[k] = -1;
   }
@@ -471,7 +516,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 
 extern "C" int tp_moe_route(const float* logits, int logit_stride, const float* correction, int experts, int top, int groups,
                             int keep, float* dense, int* ids, float* weights, int n, int score_kind, int group_best,
-                            int normalize, float sum_eps, float scale, hipStream_t s) {
+                            int normalize, float sum_eps, float scale, const float* logit_bias, hipStream_t s) {
   TP_REQUIRE(n >= 0 && experts > 0 && top > 0 && top <= experts && logit_stride >= experts, "moe_route: bad sizes");
   TP_REQUIRE(experts <= TP_WAVE * ROUTE_PER_LANE, "moe_route: %d experts exceed %d", experts, TP_WAVE * ROUTE_PER_LANE);
   TP_REQUIRE(groups <= 1 || (experts % groups == 0 && keep >= 1 && keep <= groups), "moe_route: bad groups");
@@ -479,7 +524,7 @@ extern "C" int tp_moe_route(const float* logits, int logit_stride, const float* 
   if (n == 0) return 0;
   const size_t shmem = sizeof(float) * 4 * (size_t)(experts + (groups > 1 ? groups : 1));
   hipLaunchKernelGGL(moe_route_kernel, dim3((n + 3) / 4), dim3(256), shmem, s, logits, logit_stride, correction, experts, top, groups,
-                     keep, dense, ids, weights, n, score_kind, group_best, normalize, sum_eps, scale);
+                     keep, dense, ids, weights, n, score_kind, group_best, normalize, sum_eps, scale, logit_bias);
   TP_CHECK_LAUNCH("moe_route");
   return 0;
 }
@@ -823,5 +868,75 @@ extern "C" int tp_latent_rows(const float* proj, size_t proj_stride, int q_col0,
   hipLaunchKernelGGL(latent_rows_kernel, dim3(n), dim3(256), 0, s, proj, proj_stride, q_col0, rot_col0, up, up_stride, out, heads, dim,
                      rot, vdim);
   TP_CHECK_LAUNCH("latent_rows");
+  return 0;
+}
+
+// ---- norm per head on projected rows, in place --------------------------------------------------
+// rows float32 [n, stride]: the `heads` heads of `dim` columns from col0 on become x / sqrt(mean(x^2) + eps) * w[d]
+// (one weight [dim] for all of them).  Queries and keys of an attention are two calls' worth of columns, so the entry
+// point takes two runs of heads, each with its weight.  One wave per (token, head).
+__global__ __launch_bounds__(256) void head_rmsnorm_kernel(float* __restrict__ rows, size_t stride, int col_a, int heads_a,
+                                                           const float* __restrict__ w_a, int col_b, int heads_b,
+                                                           const float* __restrict__ w_b, int dim, float eps, long pairs) {
+  const long p = (long)blockIdx.x * 4 + threadIdx.x / TP_WAVE;
+  const int lane = threadIdx.x % TP_WAVE;
+  if (p >= pairs) return;
+  const int per = heads_a + heads_b;
+  const long t = p / per;
+  const int hh = (int)(p % per);
+  float* x = rows + (size_t)t * stride + (hh < heads_a ? col_a + (size_t)hh * dim : col_b + (size_t)(hh - heads_a) * dim);
+  const float* w = hh < heads_a ? w_a : w_b;
+  float ss = 0.f;
+  for (int d = lane; d < dim; d += TP_WAVE) ss = fmaf(x[d], x[d], ss);
+  ss = wave_sum(ss);
+  const float rstd = 1.0f / sqrtf(ss / (float)dim + eps);
+  for (int d = lane; d < dim; d += TP_WAVE) x[d] = x[d] * rstd * w[d];
+}
+
+extern "C" int tp_head_rmsnorm(float* rows, size_t stride, int col_a, int heads_a, const float* w_a, int col_b, int heads_b,
+                               const float* w_b, int dim, float eps, int n, hipStream_t s) {
+  TP_REQUIRE(n >= 0 && dim > 0 && heads_a >= 0 && heads_b >= 0 && col_a >= 0 && col_b >= 0, "head_rmsnorm: bad sizes");
+  TP_REQUIRE((size_t)col_a + (size_t)heads_a * dim <= stride && (size_t)col_b + (size_t)heads_b * dim <= stride, "head_rmsnorm: rows too short");
+  TP_REQUIRE((heads_a == 0 || w_a) && (heads_b == 0 || w_b), "head_rmsnorm: a run of heads needs its weight");
+  const long pairs = (long)n * (heads_a + heads_b);
+  if (pairs == 0) return 0;
+  TP_REQUIRE((pairs + 3) / 4 < 0x7fffffffL, "head_rmsnorm: too many rows");
+  hipLaunchKernelGGL(head_rmsnorm_kernel, dim3((unsigned)((pairs + 3) / 4)), dim3(256), 0, s, rows, stride, col_a, heads_a, w_a, col_b,
+                     heads_b, w_b, dim, eps, pairs);
+  TP_CHECK_LAUNCH("head_rmsnorm");
+  return 0;
+}
+
+// ---- one vector a token into the cache, as key and as value ------------------------------------------
+// c [n, dim] goes to cache place slots[t] of keys [page, 1, page_size, dim] and of transposed values
+// [page, 1, dim, page_size]: an attention whose keys are its values reads both with the ordinary kernels.
+template <typename T>
+__global__ void vector_store_kernel(const T* __restrict__ c, const int* __restrict__ slots, T* __restrict__ k_cache,
+                                    T* __restrict__ v_cache, size_t total, int dim, int page_size) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / dim;
+  const int d = (int)(i % dim);
+  const int slot = slots[t];
+  const size_t page = slot / page_size;
+  const int off = slot % page_size;
+  const T v = c[i];
+  k_cache[(page * page_size + off) * dim + d] = v;
+  v_cache[(page * dim + d) * page_size + off] = v;
+}
+
+extern "C" int tp_vector_store(const void* c, int dt, const int* slots, void* k_cache, void* v_cache, int n, int dim, int page_size,
+                               hipStream_t s) {
+  TP_REQUIRE(n >= 0 && dim > 0 && page_size > 0, "vector_store: bad sizes");
+  const size_t total = (size_t)n * dim;
+  if (total == 0) return 0;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (dt == TP_F32)
+    hipLaunchKernelGGL(vector_store_kernel<float>, grid, dim3(256), 0, s, (const float*)c, slots, (float*)k_cache, (float*)v_cache, total, dim, page_size);
+  else if (dt == TP_BF16)
+    hipLaunchKernelGGL(vector_store_kernel<bf16_t>, grid, dim3(256), 0, s, (const bf16_t*)c, slots, (bf16_t*)k_cache, (bf16_t*)v_cache, total, dim, page_size);
+  else
+    TP_REQUIRE(false, "vector_store: unknown dtype %d", dt);
+  TP_CHECK_LAUNCH("vector_store");
   return 0;
 }

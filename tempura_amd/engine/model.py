@@ -156,6 +156,8 @@ class CausalLM:
             if state is None or self.EMBEDDING_STATE not in state:
                 raise ValueError("this model's embedding keeps per-request state: forward needs the state tensors")
             h = self.embedding.forward(tokens, ctx.positions, self.streams, ctx=ctx, state=state[self.EMBEDDING_STATE])
+        elif getattr(self.embedding, "learned", False) or getattr(self.embedding, "scale", 1.0) != 1.0:
+            h = self.embedding.forward(tokens, ctx.positions, self.streams, ctx=ctx)      # (reads the step's positions)
         elif self.streams > 1 or getattr(self.embedding, "inv_freq", None) is not None:
             h = self.embedding.forward(tokens, ctx.positions, self.streams)
         else:

@@ -839,16 +839,29 @@ portion_min_keys = 1024
 portion_scratch_limit = 256 << 20
 
 
+def fast_attention_takes(has_sink: bool, keep_first: int) -> bool:
+    """Whether the matrix-core attention kernels take a softmax with a sink and kept first keys (else the general
+    kernel runs, and no splits or partial results are prepared for them)."""
+    return not has_sink and not keep_first
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     cu_seqlens: torch.Tensor, context_lens: torch.Tensor, token_req: torch.Tensor,
                     scale: float, window: int, max_q_len: int, max_context_len: int,
-                    num_single: Optional[int] = None, dist_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    num_single: Optional[int] = None, dist_bias: Optional[torch.Tensor] = None,
+                    sink: Optional[torch.Tensor] = None, keep_first: int = 0) -> torch.Tensor:
     """q [n, heads, head_dim] over k [pages, kv_heads, page_size, head_dim] and transposed
     v [pages, kv_heads, value_dim, page_size] -> [n, heads * value_dim] (value_dim is the value cache's own; the
     matrix-core kernels take value_dim == head_dim, other sizes run the general kernel).
     ``dist_bias`` (float32 [heads, L]): added to the scaled score of a query at position p and a key at j as
-    dist_bias[head, min(p - j, L - 1)]."""
+    dist_bias[head, min(p - j, L - 1)].
+    ``sink`` (float32 [heads]): the softmax's denominator holds one more term, exp(sink[head]), without key or value.
+    ``keep_first``: under a window, the request's first ``keep_first`` keys stay visible as well."""
     if _backend is not None:
+        if sink is not None or keep_first:
+            return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
+                                            token_req, scale, window, max_q_len, max_context_len, dist_bias=dist_bias,
+                                            sink=sink, keep_first=keep_first)
         if dist_bias is not None:
             return _backend.paged_attention(q, k_cache, v_cache, block_tables, cu_seqlens, context_lens,
                                             token_req, scale, window, max_q_len, max_context_len, dist_bias=dist_bias)
@@ -879,7 +892,14 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _dev_ok(dist_bias)
         _need(dist_bias.dtype == torch.float32 and dist_bias.dim() == 2 and dist_bias.shape[0] == heads and dist_bias.shape[1] > 0,
               "paged_attention: dist_bias must be float32 [heads, L]")
+    if sink is not None:
+        _dev_ok(sink)
+        _need(sink.dtype == torch.float32 and sink.numel() == heads, "paged_attention: sink must be float32 [heads]")
+    _need(keep_first >= 0, "paged_attention: keep_first must be >= 0")
+    if not window:
+        keep_first = 0
     fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0 and vd == d
+    fast = fast and fast_attention_takes(sink is not None, keep_first)
     splits, scratch = 1, None
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
@@ -929,7 +949,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
           _ptr(cu_seqlens), _ptr(context_lens), _ptr(token_req), _ptr(out), n, r, heads, kvh, d, page_size,
           ctypes.c_float(scale), int(window), int(max_q_len), int(max_context_len), int(fast),
           int(num_single), int(splits), _ptr(scratch), int(parts), max(1, portion_min_keys // 32), _ptr(part_scratch),
-          _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1], int(vd), _stream())
+          _ptr(dist_bias), 0 if dist_bias is None else dist_bias.shape[1], int(vd), int(keep_first), _ptr(sink), _stream())
     return out
 
 
@@ -1193,31 +1213,41 @@ def fill_normal(out: torch.Tensor, seed: int, mean: float, std: float) -> torch.
 # Operations of layers with a hashed bigram embedding, norms behind the sublayers, a gated delta-rule mixer and
 # routed experts.
 
-def embed_bigram(tokens: torch.Tensor, table: torch.Tensor, bigram: torch.Tensor, positions: torch.Tensor,
+def embed_bigram(tokens: torch.Tensor, table: torch.Tensor, bigram: Optional[torch.Tensor], positions: torch.Tensor,
                  token_req: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, prev_state: torch.Tensor,
-                 num_requests: int, mul_prev: int, mul_cur: int, buckets: int) -> torch.Tensor:
-    """float32 [n, hidden] = table[token] + bigram[row], row = (previous * mul_prev + token * mul_cur) mod buckets,
+                 num_requests: int, mul_prev: int, mul_cur: int, buckets: int, scale: float = 1.0,
+                 pos_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [n, hidden] = table[token] * scale + bigram[row], row = (previous * mul_prev + token * mul_cur) mod buckets,
     and row ``buckets`` for a token at position 0.  The previous token of a run's first token is what
-    ``prev_state`` (int32 [slots, 1]) holds for the request's slot; each run's last token is left there."""
+    ``prev_state`` (int32 [slots, 1]) holds for the request's slot; each run's last token is left there.
+    ``pos_table`` ([positions, hidden], of the tables' type): its row of the token's position is added as well.
+    ``bigram`` None: no second row (and nothing is read from or left in ``prev_state``, which may be None too)."""
     if _backend is not None:
+        if scale != 1.0 or pos_table is not None:
+            return _backend.embed_bigram(tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state,
+                                         num_requests, mul_prev, mul_cur, buckets, scale, pos_table)
         return _backend.embed_bigram(tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state,
                                      num_requests, mul_prev, mul_cur, buckets)
-    _dev_ok(tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state)
+    _dev_ok(tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state, pos_table)
     n = tokens.numel()
-    _need(table.dim() == 2 and bigram.dim() == 2 and bigram.shape[1] == table.shape[1] and bigram.dtype == table.dtype,
-          "embed_bigram: tables must be [rows, hidden] of one type")
-    _need(bigram.shape[0] == buckets + 1, f"embed_bigram: the bigram table needs {buckets + 1} rows, has {bigram.shape[0]}")
+    _need(pos_table is None or (pos_table.dim() == 2 and pos_table.shape[1] == table.shape[1] and pos_table.dtype == table.dtype),
+          "embed_bigram: the position table must be [positions, hidden] of the tables' type")
+    _need(table.dim() == 2, "embed_bigram: tables must be [rows, hidden] of one type")
+    if bigram is not None:
+        _need(bigram.dim() == 2 and bigram.shape[1] == table.shape[1] and bigram.dtype == table.dtype,
+              "embed_bigram: tables must be [rows, hidden] of one type")
+        _need(bigram.shape[0] == buckets + 1, f"embed_bigram: the bigram table needs {buckets + 1} rows, has {bigram.shape[0]}")
+        _need(prev_state is not None and prev_state.dtype == torch.int32, "embed_bigram: the state must be int32")
     _i32(tokens, n, "embed tokens") if n else None
     _i32(positions, n, "embed positions") if n else None
     _i32(token_req, n, "token_req") if n else None
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
-    _need(prev_state.dtype == torch.int32, "embed_bigram: the state must be int32")
     hidden = table.shape[1]
     out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
     _call("tp_embed_bigram", _ptr(tokens), _ptr(positions), _ptr(token_req), _ptr(cu_seqlens), _ptr(state_slots), _ptr(prev_state),
           _ptr(table), _ptr(bigram), _dt(table), _ptr(out), n, int(num_requests), hidden, ctypes.c_longlong(mul_prev),
-          ctypes.c_longlong(mul_cur), ctypes.c_longlong(buckets), _stream())
+          ctypes.c_longlong(mul_cur), ctypes.c_longlong(buckets), ctypes.c_float(scale), _ptr(pos_table), _stream())
     return out
 
 
@@ -1257,16 +1287,29 @@ def norm_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
     return x
 
 
-ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
+ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "gelu_erf": 2}
 
 
-def activation(u: torch.Tensor, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
-    """Element by element: ``gelu_tanh`` (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))) or ``silu``, formed in
-    float32, as ``out_dtype``."""
+def activation(u: torch.Tensor, kind: str, out_dtype: torch.dtype, col0: int = 0, width: Optional[int] = None,
+               gate_col: Optional[int] = None) -> torch.Tensor:
+    """Element by element: ``gelu_tanh`` (0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))), ``gelu_erf``
+    (0.5 z (1 + erf(z / sqrt(2)))) or ``silu``, formed in float32, as ``out_dtype``.
+    With ``width`` (``u`` float32 rows [n, wider]): the columns col0 .. col0 + width of every row, and with ``gate_col``
+    each row's results times the sigmoid of that column of the row."""
     _need(kind in ACTIVATIONS, f"activation: {kind!r} unknown (known: {sorted(ACTIVATIONS)})")
     if _backend is not None:
+        if width is not None:
+            return _backend.activation(u, kind, out_dtype, col0, width, gate_col)
         return _backend.activation(u, kind, out_dtype)
     _dev_ok(u)
+    if width is not None:
+        _need(u.dtype == torch.float32 and u.dim() == 2 and 0 <= col0 and col0 + width <= u.shape[1] and width > 0,
+              "activation: rows must be float32 [n, wider]")
+        _need(gate_col is None or 0 <= gate_col < u.shape[1], "activation: gate column outside the rows")
+        out = torch.empty((u.shape[0], width), dtype=out_dtype, device=u.device)
+        _call("tp_activation_rows", _ptr(u), ctypes.c_size_t(u.shape[1]), int(col0), int(width), -1 if gate_col is None else int(gate_col),
+              _ptr(out), _dtcode(out_dtype), u.shape[0], ACTIVATIONS[kind], _stream())
+        return out
     out = torch.empty(u.shape, dtype=out_dtype, device=u.device)
     _call("tp_activation", _ptr(u), _dt(u), _ptr(out), _dtcode(out_dtype), ctypes.c_size_t(u.numel()), ACTIVATIONS[kind], _stream())
     return out
@@ -1276,19 +1319,25 @@ ROUTE_SCORES = {"softmax": 0, "sigmoid": 1}
 
 
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], experts: int, top: int, groups: int, keep: int,
-              score: str = "softmax", group_best: int = 1, normalize: bool = False, sum_eps: float = 0.0, scale: float = 1.0):
+              score: str = "softmax", group_best: int = 1, normalize: bool = False, sum_eps: float = 0.0, scale: float = 1.0,
+              bias: Optional[torch.Tensor] = None):
     """Router of a mixture of experts over float32 logits [n, >= experts]: s = softmax over the experts (``score``
     ``"sigmoid"``: the sigmoid of each logit by itself); an expert's choice score is s + correction (None: s); with
     ``groups`` > 1 only the experts of the ``keep`` groups (of neighbours) whose ``group_best`` largest choice scores
     add up highest can be chosen; the ``top`` best allowed experts are chosen and weigh s, with ``normalize`` divided by
     the chosen experts' sum (+ ``sum_eps``), times ``scale``.  Returns (dense float32 [n, experts] with a chosen expert's
-    weight and 0 elsewhere, ids int32 [n, top], weights [n, top])."""
+    weight and 0 elsewhere, ids int32 [n, top], weights [n, top]).  ``bias`` (float32 [experts]) is added to the logits
+    first.  (A softmax over the chosen logits alone is ``normalize`` without ``sum_eps``: the chosen experts' shares of
+    the full softmax over their sum.)"""
     _need(score in ROUTE_SCORES, f"moe_route: score {score!r} unknown")
     if _backend is not None:
+        if bias is not None:
+            return _backend.moe_route(logits, correction, experts, top, groups, keep, score, group_best, normalize, sum_eps, scale, bias)
         if (score, group_best, normalize, scale) == ("softmax", 1, False, 1.0) and correction is not None:
             return _backend.moe_route(logits, correction, experts, top, groups, keep)
         return _backend.moe_route(logits, correction, experts, top, groups, keep, score, group_best, normalize, sum_eps, scale)
-    _dev_ok(logits, correction)
+    _dev_ok(logits, correction, bias)
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == experts), "moe_route: bias must be float32 [experts]")
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[1] >= experts, "moe_route: logits must be float32 [n, experts]")
     _need(correction is None or (correction.dtype == torch.float32 and correction.numel() == experts), "moe_route: correction must be float32 [experts]")
     _need(group_best >= 1, "moe_route: group_best must be at least 1")
@@ -1298,7 +1347,7 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], experts:
     weights = torch.empty((n, top), dtype=torch.float32, device=logits.device)
     _call("tp_moe_route", _ptr(logits), logits.shape[1], _ptr(correction), int(experts), int(top), int(groups), int(keep), _ptr(dense),
           _ptr(ids), _ptr(weights), n, ROUTE_SCORES[score], int(group_best), int(bool(normalize)), ctypes.c_float(sum_eps),
-          ctypes.c_float(scale), _stream())
+          ctypes.c_float(scale), _ptr(bias), _stream())
     return dense, ids, weights
 
 
@@ -1549,3 +1598,70 @@ def latent_rows(proj: torch.Tensor, q_col0: int, rot_col0: int, up: torch.Tensor
     _call("tp_latent_rows", _ptr(proj), ctypes.c_size_t(proj.shape[1]), int(q_col0), int(rot_col0), _ptr(up), ctypes.c_size_t(up.shape[1]),
           _ptr(out), n, int(heads), int(dim), int(rot), int(vdim), _stream())
     return out
+
+
+def head_rmsnorm(rows: torch.Tensor, col_a: int, heads_a: int, weight_a: Optional[torch.Tensor], col_b: int, heads_b: int,
+                 weight_b: Optional[torch.Tensor], dim: int, eps: float) -> None:
+    """In place on float32 rows [n, wider]: each of the ``heads_a`` heads of ``dim`` columns from col_a on becomes
+    x / sqrt(mean(x^2) + eps) * weight_a (float32 [dim], one for all heads), and likewise the ``heads_b`` heads from col_b
+    on with weight_b (the queries and the keys of an attention in one launch)."""
+    if _backend is not None:
+        return _backend.head_rmsnorm(rows, col_a, heads_a, weight_a, col_b, heads_b, weight_b, dim, eps)
+    _dev_ok(rows, weight_a, weight_b)
+    _need(rows.dtype == torch.float32 and rows.dim() == 2, "head_rmsnorm: rows must be float32 [n, width]")
+    for col, heads, w in ((col_a, heads_a, weight_a), (col_b, heads_b, weight_b)):
+        _need(heads >= 0 and col >= 0 and col + heads * dim <= rows.shape[1], "head_rmsnorm: heads outside the rows")
+        _need(heads == 0 or (w is not None and w.dtype == torch.float32 and w.numel() == dim), "head_rmsnorm: weight must be float32 [dim]")
+    _call("tp_head_rmsnorm", _ptr(rows), ctypes.c_size_t(rows.shape[1]), int(col_a), int(heads_a), _ptr(weight_a), int(col_b), int(heads_b),
+          _ptr(weight_b), int(dim), ctypes.c_float(eps), rows.shape[0], _stream())
+
+
+def vector_store(c: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor) -> None:
+    """One vector a token, ``c`` [n, dim], into cache place ``slots`` of keys [pages, 1, page_size, dim] and of transposed
+    values [pages, 1, dim, page_size] (an attention whose keys are its values reads both)."""
+    if _backend is not None:
+        return _backend.vector_store(c, slots, k_cache, v_cache)
+    _dev_ok(c, slots, k_cache, v_cache)
+    _need(c.dim() == 2 and k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[1] == 1, "vector_store: bad operand ranks")
+    n, dim = c.shape
+    pages, _, page_size, d2 = k_cache.shape
+    _need(d2 == dim and tuple(v_cache.shape) == (pages, 1, dim, page_size), "vector_store: caches must be k [pages, 1, page_size, dim], v [pages, 1, dim, page_size]")
+    _need(c.dtype == k_cache.dtype == v_cache.dtype, "vector_store: vector and cache types differ")
+    _i32(slots, n, "slots") if n else None
+    _call("tp_vector_store", _ptr(c), _dt(c), _ptr(slots), _ptr(k_cache), _ptr(v_cache), n, dim, page_size, _stream())
+
+
+def mlstm_scan(proj: torch.Tensor, col0: int, i_bias: torch.Tensor, f_bias: torch.Tensor, cap: float, q_scale: float,
+               state: torch.Tensor, state_off: int, cu_seqlens: torch.Tensor, state_slots: torch.Tensor, num_requests: int,
+               heads: int, dim: int, vdim: int, norm_weight: torch.Tensor, eps: float, scale: float, out: torch.Tensor,
+               out_col0: int) -> None:
+    """The matrix-memory recurrence of an mLSTM mixer over each request's run of tokens, and its read-out as the rows
+    of the output product.  ``proj`` float32 [n, wider] holds from col0 on [q | k | v | gate | i | f] (heads * dim,
+    heads * dim, heads * vdim, heads * vdim, heads, heads columns).  With i = cap tanh((x_i + i_bias) / cap) and
+    f = logsigmoid(cap tanh((x_f + f_bias) / cap)) per head: m' = max(f + m, i); S' = e^(f + m - m') S + e^(i - m') k v^T;
+    n' likewise with k alone; o = S'^T (q * q_scale) / (max(|n' . q|, e^(-m')) + 1e-6).  Then per head o over its root
+    mean square (``eps``), times ``norm_weight`` [heads * vdim], times sigmoid(gate), times ``scale``, into columns
+    out_col0 .. of ``out``.  A request's state (float32 row of ``state`` from state_off on, heads * (vdim + 1) * (dim + 1)
+    numbers: per head the memory column by column with n as the last column, then a copy of m per column) is read and
+    left updated."""
+    if _backend is not None:
+        return _backend.mlstm_scan(proj, col0, i_bias, f_bias, cap, q_scale, state, state_off, cu_seqlens, state_slots, num_requests,
+                                   heads, dim, vdim, norm_weight, eps, scale, out, out_col0)
+    _dev_ok(proj, i_bias, f_bias, state, cu_seqlens, state_slots, norm_weight, out)
+    _need(proj.dtype == torch.float32 and proj.dim() == 2, "mlstm_scan: rows must be float32 [n, width]")
+    n = proj.shape[0]
+    width = 2 * heads * dim + 2 * heads * vdim + 2 * heads
+    _need(0 <= col0 and col0 + width <= proj.shape[1], "mlstm_scan: rows too short")
+    for b in (i_bias, f_bias):
+        _need(b.dtype == torch.float32 and b.numel() == heads, "mlstm_scan: gate biases must be float32 [heads]")
+    _need(norm_weight.dtype == torch.float32 and norm_weight.numel() == heads * vdim, "mlstm_scan: norm weight must be float32 [heads * vdim]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= state_off + heads * (vdim + 1) * (dim + 1),
+          "mlstm_scan: state rows too short")
+    _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
+    _i32(state_slots, num_requests, "state_slots")
+    _need(out.dim() == 2 and out.shape[0] == n and 0 <= out_col0 and out_col0 + heads * vdim <= out.shape[1], "mlstm_scan: output rows too short")
+    scratch = torch.empty((max(1, n * heads * (vdim + 2)),), dtype=torch.float32, device=proj.device)
+    _call("tp_mlstm_scan", _ptr(proj), proj.shape[1], int(col0), _ptr(i_bias), _ptr(f_bias), ctypes.c_float(cap), ctypes.c_float(q_scale),
+          _ptr(state), ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(scratch),
+          _ptr(norm_weight), ctypes.c_float(eps), ctypes.c_float(scale), _ptr(out), _dt(out), out.shape[1], int(out_col0), n,
+          int(num_requests), int(heads), int(dim), int(vdim), _stream())

@@ -1,6 +1,6 @@
 from .base import (Part, Mixer, BranchMixer, FeedForward, Norm, PositionEncoding, Block, CacheSpec, StateSpec,
                    WeightInfo, register_part, part_class, build_part)
-from . import norm, rope, attention, ffn, block, embedding, ssm, delta, parallel, stream, inputs  # noqa: F401  (register the built-in parts)
+from . import norm, rope, attention, ffn, block, embedding, ssm, delta, parallel, stream, inputs, mlstm  # noqa: F401  (register the built-in parts)
 from .inventory import expected_weights
 from .block import ArrangedBlock
 

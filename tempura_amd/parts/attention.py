@@ -17,6 +17,13 @@ Options beyond that, each a parameter of the part:
   n while n < B // 2, else row min(B - 1, B // 2 + floor(ln(n / (B // 2)) / ln(max_distance / (B // 2)) * (B - B // 2))).
   B is the tensor's own first dimension.
 The first two need a position encoding that does not rotate (``"none"``).
+* ``qk_norm`` (``{"eps"}``, tensors ``q_norm``, ``k_norm`` of [head_dim]): every head of q and of k is divided by its
+  root mean square and multiplied by the weight (one weight for all q heads, one for all k heads), before any rotation;
+* ``value_dim``: the values of a head have another size than its keys;
+* ``sink`` (tensor ``sink`` [heads]): the softmax's denominator holds one more term exp(sink[head]) that has no key
+  and no value;
+* ``keep_first``: under a ``window`` a query also sees the request's first ``keep_first`` keys (their pages stay held).
+The last four run without projection biases, own values, and a rows-in-float32 projection (no split norm).
 """
 from __future__ import annotations
 
@@ -86,7 +93,26 @@ class PagedAttention(Mixer):
             raise ValueError("attention: projection biases are supported together with values that are the keys")
         #: q and k come straight from the projection (biases added, keys stored as keys and as values): no rotation kernel
         self.plain_qk = self.values_are_keys
-        self.split_norm = not self.plain_qk      # (the plain projection takes finished rows only)
+        self.qk_norm = p.get("qk_norm")
+        self.value_dim = int(p.get("value_dim") or self.head_dim)
+        self.has_sink = bool(p.get("sink", False))
+        self.keep_first = int(p.get("keep_first") or 0)
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise ValueError("attention: keep_first needs a window and must not be negative")
+        #: the options that take the projection's float32 rows through kernels of their own
+        self.extended = self.qk_norm is not None or self.value_dim != self.head_dim or self.has_sink or self.keep_first > 0
+        if self.extended and (self.plain_qk or self.has_bias or self.distance_bias is not None):
+            raise ValueError("attention: qk_norm, value_dim, sink and keep_first do not combine with biases, values that are the keys "
+                             "or a distance bias")
+        self.v_dim = self.num_kv_heads * self.value_dim
+        # values wider than keys, of a size the matrix-core attention kernels take: q and the cached keys get zeros
+        # behind their own elements up to the values' size (no score changes), so that those kernels serve
+        self.key_dim = self.head_dim
+        if (dtype == torch.bfloat16 and self.head_dim < self.value_dim <= 128 and self.value_dim % 32 == 0 and self.head_dim % 2 == 0
+                and ops.fast_attention_takes(self.has_sink, self.keep_first)):
+            self.key_dim = self.value_dim
+        self.split_norm = not self.plain_qk and not self.extended      # (these projections take finished rows only)
+        self.q_norm_w = self.k_norm_w = self.sink_w = None
         self.wqkv = None
         self.wo = None
         self.q_bias = self.k_bias = self.dist_table = None
@@ -101,8 +127,15 @@ class PagedAttention(Mixer):
             w["k"]: WeightInfo((kv_dim, hidden_size)),
             w["o"]: WeightInfo((hidden_size, q_dim)),
         }
+        vd = int(p.get("value_dim") or p["head_dim"])
         if p.get("values", "own") != "keys":
-            out[w["v"]] = WeightInfo((kv_dim, hidden_size))
+            out[w["v"]] = WeightInfo((p["num_kv_heads"] * vd, hidden_size))
+        out[w["o"]] = WeightInfo((hidden_size, p["num_heads"] * vd))
+        if p.get("qk_norm") is not None:
+            out[w["q_norm"]] = WeightInfo((p["head_dim"],), "ones")
+            out[w["k_norm"]] = WeightInfo((p["head_dim"],), "ones")
+        if p.get("sink", False):
+            out[w["sink"]] = WeightInfo((p["num_heads"],))
         if p.get("bias", False):
             out[w["q_bias"]] = WeightInfo((q_dim,))
             out[w["k_bias"]] = WeightInfo((kv_dim,))
@@ -144,18 +177,27 @@ class PagedAttention(Mixer):
         # (stored tiled where the sizes allow: the products then read whole cache lines)
         self.wqkv = ops.tile_weight(torch.cat([self._to_device(t) for t in parts], dim=0).contiguous())
         self.wo = ops.tile_weight(self._to_device(get(w["o"])))
+        if self.qk_norm is not None:
+            self.q_norm_w = self._to_device(get(w["q_norm"]), torch.float32)
+            self.k_norm_w = self._to_device(get(w["k_norm"]), torch.float32)
+        if self.has_sink:
+            self.sink_w = self._to_device(get(w["sink"]), torch.float32)
         self.position.load_weights(get)
 
     def cache_spec(self):
         kind = "window" if self.window is not None else "full"
-        return CacheSpec(kind, self.num_kv_heads, self.head_dim, self.window)
+        if self.keep_first:
+            return SizedValueCacheSpec("window_keep_first", self.num_kv_heads, self.key_dim, self.window, self.value_dim, self.keep_first)
+        if self.value_dim != self.key_dim:
+            return SizedValueCacheSpec(kind, self.num_kv_heads, self.key_dim, self.window, self.value_dim)
+        return CacheSpec(kind, self.num_kv_heads, self.key_dim, self.window)
 
     def forward(self, x, ctx, cache, residual, next_norm=None):
         rot = self.position.rotary()
         q = None
         if self.plain_qk:
             q = self._project_plain(x, ctx, cache)
-        elif rot is not None and cache.writes:
+        elif rot is not None and cache.writes and not self.extended:
             rows = x.x if isinstance(x, ops.Prenormed) else x
             if ops.linear_rope_ok(x.shape[0], self.wqkv.shape[0], x.shape[1], self.head_dim, rot[1], cache.k.shape[2],
                                   rows.dtype, cache.k.dtype, isinstance(x, ops.Prenormed)):
@@ -165,7 +207,12 @@ class PagedAttention(Mixer):
                                        self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v, table)
         if q is None:
             q = self._project_and_rotate(x, ctx, cache, rot)
-        if self.dist_table is not None:
+        if self.extended:
+            a = ops.paged_attention(
+                q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
+                ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
+                ctx.num_single, sink=self.sink_w, keep_first=self.keep_first)
+        elif self.dist_table is not None:
             a = ops.paged_attention(
                 q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens,
                 ctx.token_req, self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len,
@@ -194,9 +241,30 @@ class PagedAttention(Mixer):
         rows = ops.linear(x, ops.weight_rows(self.wqkv, 0, self.q_dim), torch.float32)
         return ops.qk_store(rows, self.q_bias, None, None, self.num_heads, self.num_kv_heads, self.head_dim, None, None, self.dtype)
 
+    def _project_extended(self, x, ctx, cache, rot):
+        """q of a projection with a norm per head and/or values of their own size: the float32 rows are normed in
+        place, then rotated (if the position part rotates) and stored by the cache-write kernel."""
+        if rot is None and type(self.position).__name__ != "NoPosition":
+            raise ValueError("attention: qk_norm, value_dim, sink and keep_first need a rotary position part or none")
+        writes = cache.writes
+        w = self.wqkv if writes else ops.weight_rows(self.wqkv, 0, self.q_dim)
+        qkv = ops.linear(x, w, torch.float32)
+        if self.qk_norm is not None:
+            ops.head_rmsnorm(qkv, 0, self.num_heads, self.q_norm_w, self.q_dim, self.num_kv_heads if writes else 0, self.k_norm_w,
+                             self.head_dim, float(self.qk_norm["eps"]))
+        inv_freq, rotary_dim, factor, table = None, 0, 1.0, None
+        if rot is not None:
+            inv_freq, rotary_dim, factor = rot
+            table = self.position.table(ctx) if hasattr(self.position, "table") else None
+        return ops.rope_kv_write(qkv, ctx.positions, ctx.slot_mapping[cache.group] if writes else None, inv_freq, rotary_dim, factor,
+                                 self.num_heads, self.num_kv_heads, self.head_dim, cache.k if writes else None,
+                                 cache.v if writes else None, self.dtype, table, value_dim=self.value_dim, pad_dim=self.key_dim)
+
     def _project_and_rotate(self, x, ctx, cache, rot):
         """q (rotated, [n, heads, head_dim]) of the projection; k and v go to the cache."""
         # (with a rotary position the next kernel may add the projection's partial sums itself)
+        if self.extended:
+            return self._project_extended(x, ctx, cache, rot)
         if cache.writes:
             qkv = ops.linear(x, self.wqkv, torch.float32, partial_ok=rot is not None)
         else:
@@ -229,6 +297,8 @@ class SizedValueCacheSpec(CacheSpec):
     """Keys of ``head_dim`` and values of ``value_dim``: keys [kv_heads, page_size, head_dim] as ever, values
     transposed [kv_heads, value_dim, page_size]."""
     value_dim: int = 0
+    #: with kind ``"window_keep_first"``: the request's first keys that stay visible (and held) under the window
+    keep_first: int = 0
 
     def planes(self, page_size: int):
         return {"k": (self.num_kv_heads, page_size, self.head_dim), "v": (self.num_kv_heads, self.value_dim, page_size)}
@@ -431,3 +501,94 @@ class LatentAttention(BranchMixer):
 
 
 register_part("mixer", "latent_attention", LatentAttention)
+
+
+class LatentCacheAttention(BranchMixer):
+    """Softmax attention without positions whose cache holds ONE compressed vector a token, the latent c, from which
+    every head's keys and values are linear maps.  With H = ``num_heads``, per head D = ``head_dim`` query/key elements
+    and Dv = ``value_dim`` values, a latent of L = ``latent_dim`` and a query latent of ``query_rank``:
+
+        c_q = rmsnorm(W_dq x) * w_dq      q_h = W_uq[h] c_q                       (queries through a latent of their own)
+        c   = rmsnorm(W_dkv x) * w_dkv    k_h = W_uk[h] c    v_h = W_uv[h] c      score = (q_h . k_h) * ``scale``
+
+    causal (or under a ``window``), optionally with a ``sink`` per head in the softmax's denominator, then W_o on the
+    concatenated heads.  ``own_latent`` False: the layer has no W_dkv; its call of the run order names the cache slot of
+    the layer whose latents it reads (with its own W_uk, W_uv and everything else).
+
+    The maps are folded into the two ends: q_h . (W_uk[h] c) = (W_uk[h]^T q_h) . c and W_o[:, h] W_uv[h] (sum_j p_j c_j), so
+    the attention itself is one shared key/value head of L elements whose values are its keys, read straight from the
+    cache: a step expands nothing of what it reads, however long the context.  The folded weights W_uk[h]^T W_uq[h]
+    [H L, query_rank] and W_o[:, h] W_uv[h] [hidden, H L] are formed once at load (in float64, then rounded to the
+    compute dtype); per token they cost H L (query_rank + hidden) multiply-adds against H (D query_rank + Dv hidden) plus
+    H L (D + Dv) for the maps one after the other, which is the price of a cache and a decode step that stay small.
+
+    The columns of its input product are [dq | dkv]; it keeps no per-request state.  A page holds the latents as keys
+    [1, page_size, L] and once more transposed as values [1, L, page_size], the layout every attention kernel reads."""
+    preferred_portion_align = 8      # (the value cache is transposed: see ``PagedAttention``)
+
+    def __init__(self, spec, hidden_size, dtype, device):
+        super().__init__(spec, hidden_size, dtype, device)
+        p = spec.params
+        self.num_heads = int(p["num_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.value_dim = int(p["value_dim"])
+        self.latent_dim = int(p["latent_dim"])
+        self.query_rank = int(p["query_rank"])
+        self.scale = float(p["scale"])
+        self.norm_eps = float(p["norm_eps"])
+        self.window = p.get("window")
+        self.has_sink = bool(p.get("sink", False))
+        self.own_latent = bool(p.get("own_latent", True))
+        self.inner = self.num_heads * self.latent_dim
+        self.sink_w = None
+
+    @classmethod
+    def expected_weights(cls, spec, hidden_size):
+        p, w = spec.params, spec.weights
+        H, D, Dv, L, Q = (int(p[k]) for k in ("num_heads", "head_dim", "value_dim", "latent_dim", "query_rank"))
+        out = {w["dq"]: WeightInfo((Q, hidden_size)), w["dq_norm"]: WeightInfo((Q,), "ones"), w["uq"]: WeightInfo((H * D, Q)),
+               w["uk"]: WeightInfo((H * D, L)), w["uv"]: WeightInfo((H * Dv, L)), w["o"]: WeightInfo((hidden_size, H * Dv))}
+        if p.get("own_latent", True):
+            out[w["dkv"]] = WeightInfo((L, hidden_size))
+            out[w["dkv_norm"]] = WeightInfo((L,), "ones")
+        if p.get("sink", False):
+            out[w["sink"]] = WeightInfo((H,))
+        return out
+
+    def cache_spec(self):
+        return CacheSpec("window" if self.window is not None else "full", 1, self.latent_dim, self.window)
+
+    def load_branch(self, get):
+        w = self.spec.weights
+        H, D, Dv, L = self.num_heads, self.head_dim, self.value_dim, self.latent_dim
+        f64 = lambda name: get(w[name]).to(torch.float64)
+        uq, uk, uv, o = f64("uq").view(H, D, -1), f64("uk").view(H, D, L), f64("uv").view(H, Dv, L), f64("o").view(-1, H, Dv)
+        # queries into the latent's space: rows h L .. (h + 1) L are W_uk[h]^T W_uq[h]
+        q_fold = torch.einsum("hdl,hdq->hlq", uk, uq).reshape(H * L, -1)
+        self.w_q = ops.tile_weight(self._to_device(q_fold))
+        # and the heads' sums over the latents back out: columns h L .. (h + 1) L are W_o[:, h] W_uv[h]
+        o_fold = torch.einsum("whv,hvl->whl", o, uv).reshape(-1, H * L)
+        self.dq_norm_w = self._to_device(get(w["dq_norm"]), torch.float32)
+        rows = [get(w["dq"])]
+        if self.own_latent:
+            rows.append(get(w["dkv"]))
+            self.dkv_norm_w = self._to_device(get(w["dkv_norm"]), torch.float32)
+        if self.has_sink:
+            self.sink_w = self._to_device(get(w["sink"]), torch.float32)
+        return torch.cat([self._to_device(t) for t in rows], dim=0).contiguous(), self._to_device(o_fold)
+
+    def run(self, proj, col0, ctx, cache, out, out_col0, scale):
+        if cache.writes != self.own_latent:
+            raise ValueError("latent_cache_attention: a layer with a latent of its own writes its cache slot, one without reads another's")
+        n = proj.shape[0]
+        if cache.writes:
+            c = ops.rmsnorm_cols(proj, col0 + self.query_rank, self.latent_dim, self.dkv_norm_w, self.norm_eps, cache.k.dtype)
+            ops.vector_store(c, ctx.slot_mapping[cache.group], cache.k, cache.v)
+        cq = ops.rmsnorm_cols(proj, col0, self.query_rank, self.dq_norm_w, self.norm_eps, self.dtype)
+        q = ops.linear(cq, self.w_q, self.dtype).view(n, self.num_heads, self.latent_dim)
+        a = ops.paged_attention(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.cu_seqlens, ctx.context_lens, ctx.token_req,
+                                self.scale, int(self.window or 0), ctx.max_q_len, ctx.max_context_len, ctx.num_single, sink=self.sink_w)
+        ops.sigmoid_gate(a, None, 0, scale, out, out_col0)
+
+
+register_part("mixer", "latent_cache_attention", LatentCacheAttention)

@@ -15,6 +15,9 @@ added to every token's, chosen by a hash of the token before it and the token it
 (previous * mul_prev + token * mul_cur) mod buckets; a request's first token reads the last row.  The token before a
 step's first one is per-request state: the embedding says so with ``state_spec()`` (one int32 per request), the model
 asks for a state tensor on its behalf and hands it to ``forward``.
+
+``scale`` multiplies the token's row (not the other rows).  ``position: "learned"`` (tensor role ``position``
+[``max_positions``, hidden]) adds the row of the token's position; it combines with a bigram table.
 """
 from __future__ import annotations
 
@@ -32,8 +35,13 @@ class TokenEmbedding(Part):
         self.vocab_size = vocab_size
         self.weight = None
         kind = spec.params.get("position")
-        if kind not in (None, "sinusoid"):
-            raise ValueError(f"embedding: position {kind!r} unknown (known: sinusoid)")
+        if kind not in (None, "sinusoid", "learned"):
+            raise ValueError(f"embedding: position {kind!r} unknown (known: sinusoid, learned)")
+        self.scale = float(spec.params.get("scale", 1.0))
+        self.learned = kind == "learned"
+        self.pos_table = None
+        if self.scale != 1.0 and kind == "sinusoid":
+            raise ValueError("embedding: a scale and a sinusoidal position vector together are not supported")
         self.inv_freq = None
         if kind == "sinusoid":
             base = float(spec.params.get("position_base", 10000.0))
@@ -43,8 +51,8 @@ class TokenEmbedding(Part):
         self.bigram = spec.params.get("bigram")
         self.bigram_table = None
         if self.bigram is not None:
-            if kind is not None:
-                raise ValueError("embedding: a bigram table and a position vector together are not supported")
+            if kind == "sinusoid":
+                raise ValueError("embedding: a bigram table and a sinusoidal position vector together are not supported")
             for key in ("buckets", "mul_prev", "mul_cur"):
                 if int(self.bigram[key]) < (1 if key == "buckets" else 0):
                     raise ValueError(f"embedding: bigram {key} must be {'positive' if key == 'buckets' else 'non-negative'}")
@@ -54,12 +62,17 @@ class TokenEmbedding(Part):
         out = {spec.weights["weight"]: WeightInfo((vocab_size, hidden_size))}
         if spec.params.get("bigram") is not None:
             out[spec.weights["bigram"]] = WeightInfo((int(spec.params["bigram"]["buckets"]) + 1, hidden_size))
+        if spec.params.get("position") == "learned":
+            rows = spec.params.get("max_positions")      # (None: the tensor's own)
+            out[spec.weights["position"]] = WeightInfo((None if rows is None else int(rows), hidden_size))
         return out
 
     def load_weights(self, get):
         self.weight = self._to_device(get(self.spec.weights["weight"]))
         if self.bigram is not None:
             self.bigram_table = self._to_device(get(self.spec.weights["bigram"]))
+        if self.learned:
+            self.pos_table = self._to_device(get(self.spec.weights["position"]))
 
     def state_spec(self):
         """Per-request state of the embedding: the request's last token, for the bigram row of the next step's first."""
@@ -67,12 +80,18 @@ class TokenEmbedding(Part):
 
     def forward(self, tokens, positions=None, streams: int = 1, ctx=None, state=None):
         """int32 [tokens] -> float32 [tokens, streams * hidden]: ``streams`` copies of the residual stream."""
-        if self.bigram is not None:
+        if self.bigram is not None or self.learned or self.scale != 1.0:
             if streams != 1:
-                raise ValueError("embedding: a bigram table with several copies of the stream is not supported")
-            b = self.bigram
+                raise ValueError("embedding: a bigram table, a scale or learned positions with several copies of the stream are not supported")
+            b = self.bigram or {"mul_prev": 0, "mul_cur": 0, "buckets": 0}
+            if self.learned and getattr(ctx, "max_context_len", 0) > self.pos_table.shape[0]:
+                raise ValueError(f"embedding: position {ctx.max_context_len - 1} lies beyond the {self.pos_table.shape[0]} learned positions")
+            if self.scale == 1.0 and not self.learned:
+                return ops.embed_bigram(tokens, self.weight, self.bigram_table, ctx.positions, ctx.token_req, ctx.cu_seqlens,
+                                        ctx.state_slots, state, ctx.num_requests, int(b["mul_prev"]), int(b["mul_cur"]), int(b["buckets"]))
             return ops.embed_bigram(tokens, self.weight, self.bigram_table, ctx.positions, ctx.token_req, ctx.cu_seqlens,
-                                    ctx.state_slots, state, ctx.num_requests, int(b["mul_prev"]), int(b["mul_cur"]), int(b["buckets"]))
+                                    ctx.state_slots, state, ctx.num_requests, int(b["mul_prev"]), int(b["mul_cur"]), int(b["buckets"]),
+                                    self.scale, self.pos_table)
         if self.inv_freq is None and streams == 1:
             return ops.embed(tokens, self.weight)
         return ops.embed(tokens, self.weight, positions, self.inv_freq, streams)

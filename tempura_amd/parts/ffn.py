@@ -157,7 +157,15 @@ class RoutedExperts(FeedForward):
     Parameters of the router beyond that: ``score`` (``"softmax"`` or ``"sigmoid"``: s = sigmoid(logit), each expert by
     itself); a spec without a ``correction`` tensor has none; ``group_best`` (default 1): a group is ranked by the sum
     of that many of its largest choice scores; ``normalize``: the weights are the chosen s over their sum (plus
-    ``sum_eps``); ``scale`` multiplies the weights."""
+    ``sum_eps``); ``scale`` multiplies the weights; a ``router_bias`` tensor [experts] is added to the logits.  (A softmax
+    over the chosen logits alone is ``normalize`` with ``sum_eps`` 0.)
+
+    ``expert`` (default ``"gated"``): ``"plain"`` experts are ``down(act(up(x)))`` without a gate, ``activation`` naming the
+    function (``ops.ACTIVATIONS``; it reads the float32 sums of the up product).
+    ``shared`` (``{"intermediate_size", "activation"}``, tensor roles ``shared_up``, ``shared_down``, ``shared_gate`` [1,
+    hidden]): one more plain expert that every token uses, its output times sigmoid(w_gate . x), one number a token, added
+    to the routed sum.  The gate row rides along in the shared up product, and the gate multiplies the activations in
+    front of the down product (which is linear), not its result."""
     graph_safe = True
     returns_output = True
 
@@ -184,8 +192,20 @@ class RoutedExperts(FeedForward):
         self.weight_scale = float(p.get("scale", 1.0))
         if self.group_best < 1:
             raise ValueError("moe: group_best must be at least 1")
-        self.plain_router = (self.score, self.group_best, self.normalize, self.weight_scale) == ("softmax", 1, False, 1.0)
-        self.w_router = self.correction = None
+        self.expert_kind = str(p.get("expert", "gated"))
+        if self.expert_kind not in ("gated", "plain"):
+            raise ValueError(f"moe: expert kind {self.expert_kind!r} unknown (known: gated, plain)")
+        self.activation = str(p.get("activation", "silu"))
+        if self.expert_kind == "plain" and self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"moe: activation {self.activation!r} unknown (known: {sorted(ops.ACTIVATIONS)})")
+        self.shared = p.get("shared")
+        if self.shared is not None and str(self.shared.get("activation", "silu")) not in ops.ACTIVATIONS:
+            raise ValueError(f"moe: shared activation {self.shared.get('activation')!r} unknown")
+        self.has_router_bias = "router_bias" in spec.weights
+        self.plain_router = (self.score, self.group_best, self.normalize, self.weight_scale) == ("softmax", 1, False, 1.0) \
+            and not self.has_router_bias
+        self.w_router = self.correction = self.router_bias = None
+        self.w_shared_up = self.w_shared_down = None
         self.w13, self.w2 = [], []
 
     @classmethod
@@ -195,10 +215,19 @@ class RoutedExperts(FeedForward):
         out = {w["router"]: WeightInfo((e, hidden_size))}
         if "correction" in w:
             out[w["correction"]] = WeightInfo((e,))
+        if "router_bias" in w:
+            out[w["router_bias"]] = WeightInfo((e,))
+        gated = p.get("expert", "gated") == "gated"
         for n in range(e):
-            out[w["gate"].format(n)] = WeightInfo((i, hidden_size))
+            if gated:
+                out[w["gate"].format(n)] = WeightInfo((i, hidden_size))
             out[w["up"].format(n)] = WeightInfo((i, hidden_size))
             out[w["down"].format(n)] = WeightInfo((hidden_size, i))
+        if p.get("shared") is not None:
+            si = int(p["shared"]["intermediate_size"])
+            out[w["shared_up"]] = WeightInfo((si, hidden_size))
+            out[w["shared_down"]] = WeightInfo((hidden_size, si))
+            out[w["shared_gate"]] = WeightInfo((1, hidden_size))
         return out
 
     def load_weights(self, get):
@@ -206,34 +235,67 @@ class RoutedExperts(FeedForward):
         w = self.spec.weights
         self.w_router = ops.tile_weight(pad_rows(self._to_device(get(w["router"])), 16))
         self.correction = self._to_device(get(w["correction"]), torch.float32) if "correction" in w else None
-        self.fused = self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
+        self.router_bias = self._to_device(get(w["router_bias"]), torch.float32) if self.has_router_bias else None
+        if self.shared is not None:
+            # the gate's row behind the up rows: one product gives the activations' sums and the gate's
+            self.shared_size = int(self.shared["intermediate_size"])
+            self.w_shared_up = ops.tile_weight(pad_rows(torch.cat([self._to_device(get(w["shared_up"])),
+                                                                   self._to_device(get(w["shared_gate"])).reshape(1, -1)], dim=0), 16))
+            self.w_shared_down = ops.tile_weight(self._to_device(get(w["shared_down"])))
+        gated = self.expert_kind == "gated"
+        self.fused = gated and self.dtype == torch.bfloat16 and ops.gated_layout_ok(self.intermediate_size, self.hidden_size)
         stack, self.w2 = [], []
         for n in range(self.experts):
-            gate, up = self._to_device(get(w["gate"].format(n))), self._to_device(get(w["up"].format(n)))
-            stack.append(ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0))
+            up = self._to_device(get(w["up"].format(n)))
+            if gated:
+                gate = self._to_device(get(w["gate"].format(n)))
+                stack.append(ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0))
+            else:
+                stack.append(up)
             self.w2.append(ops.tile_weight(self._to_device(get(w["down"].format(n)))))
         # the gate/up weights of all experts are one matrix (decoding runs them as one product); an expert's own
         # are rows of it, without a copy (tiled weights are cut at multiples of sixteen rows)
-        rows = 2 * self.intermediate_size
+        rows = (2 if gated else 1) * self.intermediate_size
         stacked = torch.cat(stack, dim=0).contiguous()
         self.w13_all = ops.tile_weight(stacked) if rows % 16 == 0 else stacked
         self.w13 = [ops.weight_rows(self.w13_all, n * rows, (n + 1) * rows) for n in range(self.experts)]
 
     def _expert(self, n, rows):
+        if self.expert_kind == "plain":
+            return ops.activation(ops.linear(rows, self.w13[n], torch.float32), self.activation, self.dtype)
         if self.fused:
             return ops.linear_swiglu(rows, self.w13[n])
         return ops.swiglu(ops.linear(rows, self.w13[n], torch.float32), self.dtype)
 
+    def _add_shared(self, x, y):
+        """y += down_s(act(up_s x) * sigmoid(w_gate . x)): the expert every token uses."""
+        u = ops.linear(x, self.w_shared_up, torch.float32)
+        a = ops.activation(u, str(self.shared.get("activation", "silu")), self.dtype, 0, self.shared_size, self.shared_size)
+        ops.linear(a, self.w_shared_down, torch.float32, residual=y)
+
     def forward(self, x, ctx, residual=None):
+        if self.shared is None:
+            return self._routed(x, ctx, residual)
+        y = self._routed(x, ctx, residual)
+        self._add_shared(x, residual if residual is not None else y)
+        return y
+
+    def _routed(self, x, ctx, residual=None):
         logits = ops.linear(x, self.w_router, torch.float32)
-        if self.plain_router and self.correction is not None:
+        if self.router_bias is not None:
+            dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep, score=self.score,
+                                                group_best=self.group_best, normalize=self.normalize, sum_eps=self.sum_eps,
+                                                scale=self.weight_scale, bias=self.router_bias)
+        elif self.plain_router and self.correction is not None:
             dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep)
         else:
             dense, ids, weights = ops.moe_route(logits, self.correction, self.experts, self.top, self.groups, self.keep, score=self.score,
                                                 group_best=self.group_best, normalize=self.normalize, sum_eps=self.sum_eps,
                                                 scale=self.weight_scale)
         if getattr(ctx, "max_q_len", 1) <= 1:
-            if self.fused:
+            if self.expert_kind == "plain":
+                a = ops.activation(ops.linear(x, self.w13_all, torch.float32), self.activation, self.dtype)
+            elif self.fused:
                 a = ops.linear_swiglu(x, self.w13_all)
             else:
                 gu = ops.linear(x, self.w13_all, torch.float32)

@@ -257,7 +257,7 @@ class EmuOps:
         return q
 
     def paged_attention(self, q, k_cache, v_cache, block_tables, cu_seqlens, context_lens, token_req, scale,
-                        window, max_q_len, max_context_len, num_single=None, dist_bias=None):
+                        window, max_q_len, max_context_len, num_single=None, dist_bias=None, sink=None, keep_first=0):
         n, heads, d = q.shape
         kvh, ps = k_cache.shape[1], k_cache.shape[2]
         group = heads // kvh
@@ -275,30 +275,39 @@ class EmuOps:
             for t in range(qs, qe):
                 pos = ctx - (qe - qs) + (t - qs)
                 lo = max(0, pos - window + 1) if window > 0 else 0
+                # (the keys a query sees: the window, and under a window the request's first keep_first keys)
+                seen = torch.cat([torch.arange(0, min(keep_first, lo) if window > 0 else 0), torch.arange(lo, pos + 1)])
                 for h in range(heads):
-                    sc = (K[lo: pos + 1, h // group] @ q[t, h].double()) * scale
+                    sc = (K[seen, h // group] @ q[t, h].double()) * scale
                     if dist_bias is not None:
-                        dist = torch.clamp(pos - torch.arange(lo, pos + 1), max=dist_bias.shape[1] - 1)
+                        dist = torch.clamp(pos - seen, max=dist_bias.shape[1] - 1)
                         sc = sc + dist_bias[h].double()[dist]
-                    p = torch.softmax(sc, dim=0)
-                    out[t, h] = p @ V[lo: pos + 1, h // group]
+                    if sink is not None:
+                        p = torch.softmax(torch.cat([sc, sink[h].double().reshape(1)]), dim=0)[:-1]
+                    else:
+                        p = torch.softmax(sc, dim=0)
+                    out[t, h] = p @ V[seen, h // group]
         return out.reshape(n, heads * vd).to(q.dtype)
 
     def embed_bigram(self, tokens, table, bigram, positions, token_req, cu_seqlens, state_slots, prev_state, num_requests,
-                     mul_prev, mul_cur, buckets):
+                     mul_prev, mul_cur, buckets, scale=1.0, pos_table=None):
         out = torch.zeros(tokens.numel(), table.shape[1], dtype=torch.float64)
         cu = cu_seqlens.tolist()
         for r in range(num_requests):
             slot = int(state_slots[r])
             for t in range(cu[r], cu[r + 1]):
                 tok = int(tokens[t])
-                if int(positions[t]) == 0:
-                    row = buckets
-                else:
-                    prev = int(tokens[t - 1]) if t > cu[r] else int(prev_state[slot].reshape(-1)[0])
-                    row = (prev * mul_prev + tok * mul_cur) % buckets
-                out[t] = table[tok].double() + bigram[row].double()
-            if cu[r + 1] > cu[r]:
+                out[t] = table[tok].double() * scale
+                if bigram is not None:
+                    if int(positions[t]) == 0:
+                        row = buckets
+                    else:
+                        prev = int(tokens[t - 1]) if t > cu[r] else int(prev_state[slot].reshape(-1)[0])
+                        row = (prev * mul_prev + tok * mul_cur) % buckets
+                    out[t] += bigram[row].double()
+                if pos_table is not None:
+                    out[t] += pos_table[int(positions[t])].double()
+            if cu[r + 1] > cu[r] and bigram is not None:
                 prev_state[slot] = int(tokens[cu[r + 1] - 1])
         return out.to(torch.float32)
 
@@ -315,18 +324,23 @@ class EmuOps:
             return None
         return self.rmsnorm(h, next_weight, next_eps, out_dtype)
 
-    def activation(self, u, kind, out_dtype):
-        z = u.double()
+    def activation(self, u, kind, out_dtype, col0=0, width=None, gate_col=None):
+        z = u.double() if width is None else u.double()[:, col0: col0 + width]
         if kind == "gelu_tanh":
             v = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        elif kind == "gelu_erf":
+            v = 0.5 * z * (1.0 + torch.erf(z * 0.7071067811865476))
         else:
             v = z * torch.sigmoid(z)
+        if gate_col is not None:
+            v = v * torch.sigmoid(u.double()[:, gate_col: gate_col + 1])
         return v.to(out_dtype)
 
     def moe_route(self, logits, correction, experts, top, groups, keep, score="softmax", group_best=1, normalize=False, sum_eps=0.0,
-                  scale=1.0):
+                  scale=1.0, bias=None):
         n = logits.shape[0]
-        s = torch.softmax(logits.double()[:, :experts], dim=-1) if score == "softmax" else torch.sigmoid(logits.double()[:, :experts])
+        z = logits.double()[:, :experts] + (bias.double() if bias is not None else 0.0)
+        s = torch.softmax(z, dim=-1) if score == "softmax" else torch.sigmoid(z)
         if correction is None:
             correction = torch.zeros(experts)
         dense = torch.zeros(n, experts, dtype=torch.float32)
@@ -346,6 +360,49 @@ class EmuOps:
                 ids[t, i] = e
                 wts[t, i] = s[t, e] * factor
         return dense, ids, wts
+
+    def head_rmsnorm(self, rows, col_a, heads_a, weight_a, col_b, heads_b, weight_b, dim, eps):
+        for col, heads, w in ((col_a, heads_a, weight_a), (col_b, heads_b, weight_b)):
+            if heads:
+                x = rows[:, col: col + heads * dim].double().reshape(rows.shape[0], heads, dim)
+                x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()
+                rows[:, col: col + heads * dim] = x.reshape(rows.shape[0], heads * dim).to(torch.float32)
+
+    def vector_store(self, c, slots, k_cache, v_cache):
+        ps = k_cache.shape[2]
+        for t in range(c.shape[0]):
+            page, off = int(slots[t]) // ps, int(slots[t]) % ps
+            k_cache[page, 0, off] = c[t]
+            v_cache[page, 0, :, off] = c[t]
+
+    def mlstm_scan(self, proj, col0, i_bias, f_bias, cap, q_scale, state, state_off, cu_seqlens, state_slots, num_requests, heads, dim,
+                   vdim, norm_weight, eps, scale, out, out_col0):
+        H, D, Dv = heads, dim, vdim
+        x = proj.double()[:, col0:]
+        cu = cu_seqlens.tolist()
+        c_q, c_k, c_v, c_g, c_i, c_f = 0, H * D, 2 * H * D, 2 * H * D + H * Dv, 2 * H * D + 2 * H * Dv, 2 * H * D + 2 * H * Dv + H
+        n_state = H * (Dv + 1) * D
+        for r in range(num_requests):
+            slot = int(state_slots[r])
+            row = state[slot, state_off: state_off + n_state + H * (Dv + 1)].double()
+            S = row[:n_state].reshape(H, Dv + 1, D).clone()      # [head, column, key channel]; the last column is n
+            m = row[n_state:].reshape(H, Dv + 1)[:, 0].clone()
+            for t in range(cu[r], cu[r + 1]):
+                q = x[t, c_q: c_q + H * D].reshape(H, D) * q_scale
+                k = x[t, c_k: c_k + H * D].reshape(H, D)
+                v = torch.cat([x[t, c_v: c_v + H * Dv].reshape(H, Dv), torch.ones(H, 1, dtype=torch.float64)], dim=1)
+                i_log = cap * torch.tanh((x[t, c_i: c_i + H] + i_bias.double()) / cap)
+                f_log = torch.nn.functional.logsigmoid(cap * torch.tanh((x[t, c_f: c_f + H] + f_bias.double()) / cap))
+                m_new = torch.maximum(f_log + m, i_log)
+                S = torch.exp(f_log + m - m_new)[:, None, None] * S + torch.exp(i_log - m_new)[:, None, None] * v[:, :, None] * k[:, None, :]
+                m = m_new
+                read = torch.einsum("hcd,hd->hc", S, q)
+                o = read[:, :Dv] / (torch.maximum(read[:, Dv].abs(), torch.exp(-m)) + 1e-6)[:, None]
+                o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
+                o = o.reshape(H * Dv) * norm_weight.double() * torch.sigmoid(x[t, c_g: c_g + H * Dv]) * scale
+                out[t, out_col0: out_col0 + H * Dv] = o.to(out.dtype)
+            state[slot, state_off: state_off + n_state] = S.reshape(-1).to(torch.float32)
+            state[slot, state_off + n_state: state_off + n_state + H * (Dv + 1)] = m[:, None].expand(H, Dv + 1).reshape(-1).to(torch.float32)
 
     def moe_plan(self, ids, experts):
         flat = ids.reshape(-1).tolist()
