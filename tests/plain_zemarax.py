@@ -212,3 +212,19 @@ def forward(cfg, W, tokens, layers_out=None):
             layers_out.append(x.clone())
     x = norm_around_zero(x, W["final.norm"], eps)
     return (x @ W["head"].T) * float(cfg.get("logit_scale", 1.0))
+
+
+def greedy(config, weights, prompt, n_new):
+    """The tokens that greedy decoding appends to ``prompt`` (the whole sequence is run anew for every token)."""
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(torch.argmax(forward(config, weights, toks)[-1])))
+    return toks[len(prompt):]
+
+
+def logit_error(got, ref):
+    """Largest difference between two sets of logits after taking each row's mean off, relative to the reference's
+    spread."""
+    g, r = got.to(F64).cpu(), ref.to(F64)
+    d = (g - g.mean(-1, keepdim=True)) - (r - r.mean(-1, keepdim=True))
+    return float(d.abs().max() / r.std())
