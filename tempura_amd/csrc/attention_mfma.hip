@@ -96,8 +96,16 @@ struct AttnArgs {
   // take (4, 2 or 1); with 2 or 1 the waves left over take further query tiles of the same heads, so that a model
   // with as many key heads as heads has no idle waves
   int heads_per_block;
+  // a sink per head: the softmax's denominator holds one more term, exp(sink[head]), without key or value (nullptr:
+  // none).  Whoever normalises a row adds it once: the kernel that writes the row, or the kernel that combines its parts.
+  const float* sink;
 };
 #define PART_STRIDE(D) ((D) + 4)
+// the sink's share of a denominator that is relative to the maximum m (scores and m are in units of log 2): 2^(sink *
+// log2(e) - m); a sink far above m makes the sum infinite and the row zero, which is its limit
+__device__ inline float sink_term(const float* sink, int head, float m) {
+  return sink != nullptr ? __builtin_amdgcn_exp2f(fmaf(sink[head], 1.4426950408889634f, -m)) : 0.f;
+}
 
 // The keys and values of one step of 32 keys, as MFMA operand fragments.
 template <int D>
@@ -406,7 +414,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_
     float lt = l[nq];
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
-    const float inv = 1.0f / lt;
+    const float inv = 1.0f / (lt + sink_term(a.sink, head, m[nq]));
     const int qi = q0 + nq * 16 + c;
     if (qi < q_len) {
       bf16_t* orow = a.out + ((size_t)(q_start + qi) * a.n_heads + head) * D;
@@ -768,7 +776,7 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     float lt = l[nq];
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
-    const float inv = 1.0f / lt;
+    const float inv = 1.0f / (lt + sink_term(a.sink, head, m[nq]));   // (used by rows this block writes itself)
     const int qi = q0 + nq * 16 + c;
     if (qi < q_len && my_parts > 1) {
       float* pr = a.portion_scratch + (((size_t)(q_start + qi) * a.n_heads + head) * a.portion_splits + part) * PART_STRIDE(D);
@@ -867,6 +875,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
       lsum += f * red_l[w][col];
     }
     if (a.num_splits == 1) {  // nothing to combine: this is the answer
+      lsum += sink_term(a.sink, kvh * group + h0 + col, mu);
       a.out[((size_t)q_start * a.n_heads + (kvh * group + h0 + col)) * D + d] = float_to_bf16(acc / lsum);
       continue;
     }
@@ -887,7 +896,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restrict__ scratch,
                                                           const int* __restrict__ cu_seqlens,
                                                           bf16_t* __restrict__ out, int n_heads, int D,
-                                                          int num_splits) {
+                                                          int num_splits, const float* __restrict__ sink) {
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int q_start = cu_seqlens[r];
   if (cu_seqlens[r + 1] - q_start != 1) return;
@@ -900,7 +909,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(const float* __restric
   const float mg = wave_max(ms);
   const float mu = (mg == -INFINITY) ? 0.f : mg;
   const float ws = __builtin_amdgcn_exp2f(ms - mu);  // 0 for lanes without a split
-  const float inv = 1.0f / wave_sum(ws * ls);
+  const float inv = 1.0f / (wave_sum(ws * ls) + sink_term(sink, h, mu));
   // (every lane runs every turn of these loops, also where the head size is no multiple of 64: a lane that sat
   // out a turn could not hand its split's weight to the others, and with more than 32 splits of a head size of
   // 32 or 96 the lanes that hold the later splits' weights would sit out)
@@ -929,7 +938,8 @@ __global__ __launch_bounds__(64) void attn_combine_rows_kernel(const float* __re
                                                                const int* __restrict__ context_lens,
                                                                const int* __restrict__ token_req,
                                                                bf16_t* __restrict__ out, int n_heads, int D,
-                                                               int max_parts, int min_steps, int window, int skip_single) {
+                                                               int max_parts, int min_steps, int window, int skip_single,
+                                                               const float* __restrict__ sink) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int r = token_req[t];
   const int q_start = cu_seqlens[r], q_len = cu_seqlens[r + 1] - q_start;
@@ -950,7 +960,7 @@ __global__ __launch_bounds__(64) void attn_combine_rows_kernel(const float* __re
   const float mg = wave_max(ms);
   const float mu = (mg == -INFINITY) ? 0.f : mg;
   const float ws = __builtin_amdgcn_exp2f(ms - mu);  // 0 for lanes without a part
-  const float inv = 1.0f / wave_sum(ws * ls);
+  const float inv = 1.0f / (wave_sum(ws * ls) + sink_term(sink, h, mu));
   for (int d0 = 0; d0 < D; d0 += 64) {      // (every lane runs every turn: see attn_combine_kernel)
     const int d = min(d0 + lane, D - 1);
     float acc = 0.f;
@@ -977,7 +987,7 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     if (a.num_splits > 1) {
       const dim3 cgrid(n_req, a.n_heads);
       hipLaunchKernelGGL(attn_combine_kernel, cgrid, dim3(64), 0, s, a.scratch, a.cu_seqlens, a.out, a.n_heads, D,
-                         a.num_splits);
+                         a.num_splits, a.sink);
     }
   }
   if (has_multi) {
@@ -1019,7 +1029,7 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
         hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), sgrid, dim3(256), 0, s, a, skip);
         hipLaunchKernelGGL(attn_combine_rows_kernel, dim3(n_tokens, a.n_heads), dim3(64), 0, s, a.portion_scratch,
                            a.cu_seqlens, a.context_lens, a.token_req, a.out, a.n_heads, D, a.portion_splits,
-                           a.portion_min_steps, a.window, skip);
+                           a.portion_min_steps, a.window, skip, a.sink);
         return 0;
       }
     }
@@ -1065,7 +1075,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int portion_splits, int portion_min_steps, float* portion_scratch, const float* dist_bias,
                             int bias_len, int keep_first, const float* sink, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
-  if (keep_first > 0 || sink != nullptr) return -1;   // (kept first keys and a sink run the general kernel)
+  if (keep_first > 0) return -1;   // (kept first keys under a window run the general kernel)
   if (portion_min_steps < 1) return -1;
   if (portion_splits < 1 || portion_splits > 64 || (portion_splits > 1 && (portion_scratch == nullptr || token_req == nullptr))) return -1;
   if ((long)n_req * portion_splits > 65535) return -1;
@@ -1097,6 +1107,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
   a.dist_bias = dist_bias;
   a.bias_len = bias_len;
   a.heads_per_block = 4;
+  a.sink = sink;
   if (dist_bias != nullptr && bias_len <= 0) return -1;
   a.scale_log2 = scale * 1.4426950408889634f;
   switch (head_dim) {

@@ -841,8 +841,8 @@ portion_scratch_limit = 256 << 20
 
 def fast_attention_takes(has_sink: bool, keep_first: int) -> bool:
     """Whether the matrix-core attention kernels take a softmax with a sink and kept first keys (else the general
-    kernel runs, and no splits or partial results are prepared for them)."""
-    return not has_sink and not keep_first
+    kernel runs, and no splits or partial results are prepared for them): a sink yes, kept first keys under a window no."""
+    return not keep_first
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,

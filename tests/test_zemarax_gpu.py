@@ -163,7 +163,8 @@ def _paged(ctx_lens, kvh, d, vd, ps, dtype, g, spare=3):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,kvh,d,vd,window,keep", [(4, 2, 12, 10, 9, 3), (1, 1, 20, 28, 16, 0), (3, 3, 6, 6, 5, 11), (4, 2, 64, 64, 40, 8),
-                                                      (8, 1, 96, 96, 0, 0), (2, 1, 64, 80, 33, 17), (4, 4, 32, 32, 64, 64)])
+                                                      (8, 1, 96, 96, 0, 0), (2, 1, 64, 80, 33, 17), (4, 4, 32, 32, 64, 64), (4, 2, 128, 128, 50, 0),
+                                                      (16, 1, 64, 64, 0, 0), (2, 2, 32, 32, 0, 0)])
 def test_attention_with_a_sink_and_kept_first_keys(dtype, heads, kvh, d, vd, window, keep):
     """Portions behind cached prefixes and single tokens in one batch; with and without the sink; large sinks too."""
     ops = _ops()
@@ -177,8 +178,16 @@ def test_attention_with_a_sink_and_kept_first_keys(dtype, heads, kvh, d, vd, win
     tol = 2e-5 if dtype == torch.float32 else 1.6e-2
     for sink in (None, torch.randn(heads, generator=g) + 1.0, torch.tensor([9.0] * heads), torch.tensor([-40.0] * heads)):
         want = emu.paged_attention(q, k, v, bt, cu, cl, token_req, 0.3, window, max(q_lens), max(ctx_lens), None, None, sink, keep)
-        got = ops.paged_attention(q.to(DEV), k.to(DEV), v.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), token_req.to(DEV), 0.3, window,
-                                  max(q_lens), max(ctx_lens), 0, sink=None if sink is None else sink.to(DEV), keep_first=keep)
+        for singles in (0, 2):      # (the single tokens as portions of one, and through the kernels for decoding)
+            got = ops.paged_attention(q.to(DEV), k.to(DEV), v.to(DEV), bt.to(DEV), cu.to(DEV), cl.to(DEV), token_req.to(DEV), 0.3, window,
+                                      max(q_lens), max(ctx_lens), singles, sink=None if sink is None else sink.to(DEV), keep_first=keep)
+            _close(got, want, tol)
+        # a step of single tokens only (split over the context and combined, where the matrix-core kernels serve)
+        q1 = (torch.randn(5, heads, d, generator=g) * 2).to(dtype)
+        cu1, tr1, _ = _batch([1] * 5, [0] * 5)
+        want = emu.paged_attention(q1, k, v, bt, cu1, cl, tr1, 0.3, window, 1, max(ctx_lens), None, None, sink, keep)
+        got = ops.paged_attention(q1.to(DEV), k.to(DEV), v.to(DEV), bt.to(DEV), cu1.to(DEV), cl.to(DEV), tr1.to(DEV), 0.3, window, 1,
+                                  max(ctx_lens), 5, sink=None if sink is None else sink.to(DEV), keep_first=keep)
         _close(got, want, tol)
     if window:
         without = emu.paged_attention(q, k, v, bt, cu, cl, token_req, 0.3, window, max(q_lens), max(ctx_lens), None, None, None, 0)
@@ -413,8 +422,6 @@ def test_a_far_latent_decides_on_the_gpu(tmp_path, dtype="float32"):
         at += c
     rows += [runner.step([StepEntry("r", [t], [0])]).cpu() for t in toks[at:]]
     assert plain.logit_error(torch.cat(rows), ref) < SHARP_TOL
-    # the premise: the far keys matter (a context cut to its last 64 tokens gives other logits at the end)
-    assert plain.logit_error(plain.forward(cfg, W, toks[-64:])[-8:], ref[-8:]) > 0.05
 
 
 def test_long_decoding_through_a_captured_step(dirs):
