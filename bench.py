@@ -58,7 +58,7 @@ def parse_args():
     ap.add_argument("--mixed-chunk", type=int, default=512)
     ap.add_argument("--mixed-temperature", type=float, default=0.0, help="0: greedy; above: seeded sampling with top-k 50")
     ap.add_argument("--decode-target-blocks", type=int, default=None, help="tuning: blocks the split decode attention aims at")
-    ap.add_argument("--design", default=None, choices=["mifutar", "bomotar", "golavik"],
+    ap.add_argument("--design", default=None, choices=["mifutar", "bomotar", "golavik", "zemarax"],
                     help="instead of the headline: prefill and decode throughput of this design at layer sizes of real models, "
                          "beside Llama layers of equal size, with the time of every kernel entry point")
     ap.add_argument("--design-sizes", default="2048,4096", help="model widths of --design (comma separated)")
@@ -84,9 +84,16 @@ def design_bench(args) -> int:
     (three quarters of a head unrotated, a quarter rotated, values as wide as the whole key, a latent of 512, window
     1,024) and a channel delta rule again, each with eight experts of a quarter of the dense width, two a token out of
     two of four groups, a norm in eight parts and four taps on the inputs; it stands beside the Bomotar model and the
-    Llama layers.  Prints one JSON line."""
+    Llama layers.  A Zemarax model here has layers of an mLSTM (width / 128 heads of 128 x 128), a latent attention of
+    the Llama layer's heads (a latent of 128, a query latent of width / 4), a windowed attention of the Llama layer's
+    heads with a norm per head (window 1,024 keeping the first 64 tokens) and a latent attention that reads the second
+    layer's latents, every attention with a sink; feed-forwards alternate between a dense one and eight ungated experts
+    of a quarter of its width, two a token, with a shared expert; it stands beside the Bomotar model (the closest: norms
+    around every sublayer, a matrix recurrence, a bigram embedding, routed experts) and the Llama layers.
+    Prints one JSON line."""
     import torch
     from tempura_amd.config import BomotarConfig, GolavikConfig, LlamaConfig, MifutarConfig
+    from tempura_amd.config.zemarax import ZemaraxConfig
     from tempura_amd.engine import Engine
     from tempura_amd.engine.loading import random_model
     from tempura_amd.engine.runner import StepEntry
@@ -133,6 +140,21 @@ def design_bench(args) -> int:
         ls = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": moe} for i in range(layers)]
         return GolavikConfig.from_dict({"architecture": "Golavik", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 8},
                                         "canon": {"taps": 4}, "layers": ls, "max_positions": 8192})
+
+    def zemarax_config(width, ff, heads, dim, kv, layers):
+        mlstm = {"heads": width // 128, "dim": 128, "vdim": 128, "gate_cap": 15.0}
+        latent = {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": 128, "q_rank": width // 4, "scale": dim ** -0.5}
+        attn = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": window, "keep_first": 64}}
+        dense = {"kind": "dense", "ff": ff}
+        moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2}, "shared": {"ff": ff // 4}}
+        ls = []
+        for i in range(layers):
+            kind = ("mlstm", "latent_attention", "attention", "latent_attention")[i % 4]
+            mixer = {"mlstm": mlstm, "attention": attn}.get(kind) or (dict(latent, kv_from=i - 2) if i % 4 == 3 else latent)
+            ls.append({"type": kind, "mixer": mixer, "mlp": moe if i % 2 else dense})
+        return ZemaraxConfig.from_dict({"architecture": "Zemarax", "vocab": vocab, "width": width, "max_positions": 8192, "logit_scale": 1.0,
+                                        "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+                                        "layers": ls})
 
     def llama_config(width, ff, heads, dim, kv, layers):
         return LlamaConfig(width, ff, layers, heads, kv, dim, vocab, 8192, 1e-5, 500000.0, None, False,
@@ -193,6 +215,9 @@ def design_bench(args) -> int:
         if design == "golavik":
             models = [("golavik", golavik_config(width, ff, heads, dim, kv, args.design_layers)),
                       ("bomotar", bomotar_config(width, ff, heads, dim, kv, args.design_layers)), models[1]]
+        if design == "zemarax":
+            models = [("zemarax", zemarax_config(width, ff, heads, dim, kv, args.design_layers)),
+                      ("bomotar", bomotar_config(width, ff, heads, dim, kv, args.design_layers)), models[1]]
         chosen = [m for m in args.design_models.split(",") if m]
         for name, cfg in [m for m in models if not chosen or m[0] in chosen]:
             say(f"{name} width {width}: building")
@@ -208,7 +233,8 @@ def design_bench(args) -> int:
                       "data": "synthetic", "vs_baseline": None,
                       "config": {"design": {"mifutar": "Mifutar beside Llama layers of equal size",
                                             "bomotar": "Bomotar beside Mifutar and Llama layers of equal size",
-                                            "golavik": "Golavik beside Bomotar and Llama layers of equal size"}[design],
+                                            "golavik": "Golavik beside Bomotar and Llama layers of equal size",
+                                            "zemarax": "Zemarax beside Bomotar and Llama layers of equal size"}[design],
                                  "layers": args.design_layers, "prompt": T, "decode_batch": batch,
                                  "window": window if design == "mifutar" else None}, "points": points}))
     return 0

@@ -99,6 +99,9 @@ struct AttnArgs {
   // a sink per head: the softmax's denominator holds one more term, exp(sink[head]), without key or value (nullptr:
   // none).  Whoever normalises a row adds it once: the kernel that writes the row, or the kernel that combines its parts.
   const float* sink;
+  // under a window, the request's first keep_first keys stay visible (0: none).  Only the kernels that load keys and
+  // values per wave take it (their steps before the window's first are the kept keys'); the host sends such calls there.
+  int keep_first;
 };
 #define PART_STRIDE(D) ((D) + 4)
 // the sink's share of a denominator that is relative to the maximum m (scores and m are in units of log 2): 2^(sink *
@@ -218,7 +221,7 @@ __device__ inline void attn_softmax(const AttnArgs& a, int j0, const f32x4_t (&s
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = j0 + 8 * g + 4 * t + r;
-          v[t * 4 + r] = (key <= hi && key >= lo) ? s[nq][t][r] : -INFINITY;
+          v[t * 4 + r] = (key <= hi && (key >= lo || key < a.keep_first)) ? s[nq][t][r] : -INFINITY;
         }
     } else {
 #pragma unroll
@@ -407,6 +410,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int skip_
   int first = 0;
   if (a.window > 0) first = max(0, pos0 + q0 - a.window + 1) & ~31;
   const float* bias_row = BIAS ? a.dist_bias + (size_t)head * a.bias_len : nullptr;
+  // the kept first keys that lie before the window's first step (keys are visited in ascending order either way)
+  const int kept_end = min(first, (a.keep_first + 31) & ~31);
+  for (int j0 = 0; j0 < kept_end; j0 += 32) attn_step<D, NQ, BIAS>(a, table, kvh, ctx, j0, qf, qpos, m, l, o, bias_row);
   for (int j0 = first; j0 <= last_pos; j0 += 32) attn_step<D, NQ, BIAS>(a, table, kvh, ctx, j0, qf, qpos, m, l, o, bias_row);
 
 #pragma unroll
@@ -839,13 +845,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(AttnArgs a) {
 
   int first = 0;
   if (a.window > 0) first = max(0, pos - a.window + 1) & ~31;
-  const int steps = (ctx - first + 31) / 32;
+  // steps of 32 keys: those of the kept first keys that lie before the window's first step, then the window's
+  const int kept_steps = min(first, (a.keep_first + 31) & ~31) / 32;
+  const int steps = kept_steps + (ctx - first + 31) / 32;
   const int per_split = (steps + a.num_splits - 1) / a.num_splits;
   const int s_begin = blockIdx.z * per_split, s_end = min(steps, s_begin + per_split);
   // (Fetching the next step's fragments while this one is computed was measured: the doubled
   // fragment registers halve the occupancy and the kernel gets slower, not faster.)
   const float* bias_row = BIAS ? a.dist_bias + (size_t)head * a.bias_len : nullptr;   // (a column is a head)
-  for (int s = s_begin + wave; s < s_end; s += 4) attn_step<D, 1, BIAS>(a, table, kvh, ctx, first + s * 32, qf, qpos, m, l, o, bias_row);
+  for (int s = s_begin + wave; s < s_end; s += 4)
+    attn_step<D, 1, BIAS>(a, table, kvh, ctx, s < kept_steps ? s * 32 : first + (s - kept_steps) * 32, qf, qpos, m, l, o, bias_row);
 
   // merge the four waves (fixed order), then write this split's partial
   float lt = l[0];
@@ -1023,7 +1032,7 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
       return 0;
     }
     if constexpr (D == 32 || D == 64 || D == 128) {
-      if (a.portion_splits > 1 && g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
+      if (a.portion_splits > 1 && g_attn_tune != 1 && a.keep_first == 0 && a.page_shift >= 4 && a.page_size >= 512 / D) {
         // few query blocks under a long context: the keys of each are split over blocks (of 32 query rows)
         const dim3 sgrid((max_q_len + 31) / 32, kv_groups, n_req * a.portion_splits);
         hipLaunchKernelGGL((attn_prefill_lds_kernel<D, 2>), sgrid, dim3(256), 0, s, a, skip);
@@ -1037,7 +1046,7 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
-      if (g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
+      if (g_attn_tune != 1 && a.keep_first == 0 && a.page_shift >= 4 && a.page_size >= 512 / D) {
         if (group <= 2) {
           // one or two heads a key group: a block takes them all and 4 / group query tiles of each (its four waves
           // share the keys and values of 64 or 128 rows instead of three or two of them idling)
@@ -1075,7 +1084,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
                             int portion_splits, int portion_min_steps, float* portion_scratch, const float* dist_bias,
                             int bias_len, int keep_first, const float* sink, hipStream_t s) {
   if (head_dim % 32 != 0 || head_dim > 128 || page_size % 8 != 0) return -1;
-  if (keep_first > 0) return -1;   // (kept first keys under a window run the general kernel)
+  if (keep_first > 0 && (dist_bias != nullptr || window <= 0)) return -1;
   if (portion_min_steps < 1) return -1;
   if (portion_splits < 1 || portion_splits > 64 || (portion_splits > 1 && (portion_scratch == nullptr || token_req == nullptr))) return -1;
   if ((long)n_req * portion_splits > 65535) return -1;
@@ -1108,6 +1117,7 @@ int tp_paged_attention_fast(const void* q, const void* k_cache, const void* v_ca
   a.bias_len = bias_len;
   a.heads_per_block = 4;
   a.sink = sink;
+  a.keep_first = window > 0 ? keep_first : 0;
   if (dist_bias != nullptr && bias_len <= 0) return -1;
   a.scale_log2 = scale * 1.4426950408889634f;
   switch (head_dim) {

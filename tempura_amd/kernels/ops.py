@@ -841,8 +841,9 @@ portion_scratch_limit = 256 << 20
 
 def fast_attention_takes(has_sink: bool, keep_first: int) -> bool:
     """Whether the matrix-core attention kernels take a softmax with a sink and kept first keys (else the general
-    kernel runs, and no splits or partial results are prepared for them): a sink yes, kept first keys under a window no."""
-    return not keep_first
+    kernel runs, and no splits or partial results are prepared for them): both (kept first keys by the kernels that
+    load keys and values per wave, whose portions are never split over blocks)."""
+    return True
 
 
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
@@ -899,7 +900,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if not window:
         keep_first = 0
     fast = allow_fast_attention and q.dtype == torch.bfloat16 and d % 32 == 0 and d <= 128 and page_size % 8 == 0 and vd == d
-    fast = fast and fast_attention_takes(sink is not None, keep_first)
+    fast = fast and fast_attention_takes(sink is not None, keep_first) and not (keep_first and dist_bias is not None)
     splits, scratch = 1, None
     if fast and num_single > 0:
         # enough blocks to fill 256 CUs, but at least 128 keys per block
@@ -933,7 +934,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             scratch = torch.empty((r * heads * splits * (d + 2),), dtype=torch.float32, device=q.device)
     parts, part_scratch = 1, None
     # (the kernel with a distance bias does not split a portion's keys)
-    if fast and dist_bias is None and num_single < r and d in (32, 64, 128) and page_size & (page_size - 1) == 0 and page_size >= max(8, 512 // d):
+    if fast and dist_bias is None and not keep_first and num_single < r and d in (32, 64, 128) and page_size & (page_size - 1) == 0 and page_size >= max(8, 512 // d):
         # Few query blocks under a long context (a portion of a prompt behind a long cached prefix): the keys of
         # every portion are split over blocks until the chip is full (T = 512 behind 7,680 keys: 219 -> 137 us).
         q_blocks = -(-(n - num_single) // 32) + (r - num_single)
