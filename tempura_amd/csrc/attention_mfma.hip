@@ -99,8 +99,9 @@ struct AttnArgs {
   // a sink per head: the softmax's denominator holds one more term, exp(sink[head]), without key or value (nullptr:
   // none).  Whoever normalises a row adds it once: the kernel that writes the row, or the kernel that combines its parts.
   const float* sink;
-  // under a window, the request's first keep_first keys stay visible (0: none).  Only the kernels that load keys and
-  // values per wave take it (their steps before the window's first are the kept keys'); the host sends such calls there.
+  // under a window, the request's first keep_first keys stay visible (0: none): the steps of the kept keys that lie
+  // before the window's first step come first, and the masks let a key pass that is kept.  (Not in the kernels with a
+  // bias by distance, and never together with portions whose keys are split over blocks: the host sees to both.)
   int keep_first;
 };
 #define PART_STRIDE(D) ((D) + 4)
@@ -279,7 +280,7 @@ __device__ inline void attn_softmax_max(const AttnArgs& a, int j0, const f32x4_t
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = j0 + 8 * g + 4 * t + r;
-          v[nq][t * 4 + r] = (key <= hi && key >= lo) ? s[nq][t][r] : -INFINITY;
+          v[nq][t * 4 + r] = (key <= hi && (key >= lo || key < a.keep_first)) ? s[nq][t][r] : -INFINITY;
         }
     } else {
 #pragma unroll
@@ -536,6 +537,10 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     first += s_begin * 32;
     nsteps = s_end - s_begin;
   }
+  // kept first keys (never together with parts): their steps come first, then the window's; step s starts at key0(s)
+  const int kept_steps = (a.keep_first > 0 && my_parts == 1) ? min(first, (a.keep_first + 31) & ~31) / 32 : 0;
+  nsteps += kept_steps;
+  auto key0 = [&](int step) { return step < kept_steps ? step * 32 : first + (step - kept_steps) * 32; };
   const int qpos_min = pos0 + min(q0, q_len - 1);   // the earliest query of this wave
   if constexpr (BIAS) {
     for (int i = lane; i < a.bias_len; i += 64) bias_lds[wave * ATTN_BIAS_LDS + i] = a.dist_bias[(size_t)head * a.bias_len + i];
@@ -586,12 +591,12 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
   // the pages of the two halves of the step that is issued next (the second clamped to the last key that exists)
   int pp0 = 0, pp1 = 0;
   auto pages_of = [&](int step) {
-    const int j0 = first + step * 32;
+    const int j0 = key0(step);
     pp0 = ctab[j0 >> psh];
     pp1 = ctab[min(j0 + 16, (ctx - 1) & ~7) >> psh];
   };
   auto issue = [&](int step, int stage) {
-    const int j0 = first + step * 32;
+    const int j0 = key0(step);
     unsigned char* buf = stages + stage * STAGE;
     if (j0 + 32 <= ctx) {   // all 32 keys exist
 #pragma unroll
@@ -696,7 +701,7 @@ __global__ __launch_bounds__(256, OCC) void attn_prefill_lds_kernel(AttnArgs a, 
     float alpha[NQ];
     bool moved[NQ];
     u32x4_t vv[D / 16];
-    const int j0 = first + s * 32;
+    const int j0 = key0(s);
     const bool plain_step = j0 + 31 <= qpos_min && (a.window <= 0 || j0 >= last_mine - a.window + 1);
 #define ATTN_RV(dt) if constexpr (dt < D / 16) vv[dt] = attn_lds_read<(dt >> 1) * 2048 + (dt & 1) * 256>(base + vaddr)
 #define ATTN_BODY(NEXT, MASK)                                                                          \
@@ -1046,7 +1051,7 @@ static int launch_all(AttnArgs a, int n_tokens, int n_req, int max_q_len, int nu
     const dim3 grid((max_q_len + rows - 1) / rows, kv_groups, n_req);
     if constexpr (D == 32 || D == 64 || D == 128) {
       // (a key load covers 512 / D rows, which must lie in one page)
-      if (g_attn_tune != 1 && a.keep_first == 0 && a.page_shift >= 4 && a.page_size >= 512 / D) {
+      if (g_attn_tune != 1 && a.page_shift >= 4 && a.page_size >= 512 / D) {
         if (group <= 2) {
           // one or two heads a key group: a block takes them all and 4 / group query tiles of each (its four waves
           // share the keys and values of 64 or 128 rows instead of three or two of them idling)

@@ -10,8 +10,11 @@
 // read-outs by row permutes.  Every column carries a copy of m in the state (no column reads what another writes).
 // The division, which needs the normaliser's column, is left to the kernel behind the scan.
 //
-// Gates: i = cap tanh((x_i + b_i) / cap), f = logsigmoid(cap tanh((x_f + b_f) / cap)).  m over a chunk of tokens comes
-// from two prefix scans over the chunk's lanes (F_t = sum_(s<=t) f_s, m_t = F_t + max(m_0, max_(s<=t) (i_s - F_s))):
+// Gates: i = cap tanh((x_i + b_i) / cap), f = logsigmoid(cap tanh((x_f + b_f) / cap)).  A kernel in front of the scan (a
+// wave per request and head, 64 tokens a turn) forms them, the running maximum and, per token, the decay
+// keep = e^(f + m - m') and the input weight put = e^(i - m'): inside the scan they would stand in every chunk's way
+// (a chain of lane exchanges and transcendental functions between two barriers while the other waves wait).  m over
+// 64 tokens comes from two prefix scans over the lanes (F_t = sum_(s<=t) f_s, m_t = F_t + max(m_0, max_(s<=t) (i_s - F_s))):
 // the read-out does not depend on which m is used as long as the decay, the input weight and the floor e^(-m') use
 // the same one, so the order of these sums changes rounding only.
 //
@@ -27,6 +30,8 @@ struct MlstmArgs {
   int stride, q_col, k_col, v_col, i_col, f_col;
   const float* i_bias;     // [heads]
   const float* f_bias;     // [heads]
+  float* keep;             // [n, heads] e^(f + m - m')
+  float* put;              // [n, heads] e^(i - m')
   float cap, q_scale;
   float* state;
   size_t state_stride, state_off;
@@ -40,6 +45,48 @@ struct MlstmArgs {
 
 __device__ inline float m_logsigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
+// grid: (requests, heads); block: one wave.
+__global__ __launch_bounds__(64) void mlstm_gates_kernel(MlstmArgs a) {
+  const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int start = a.cu_seqlens[r], len = a.cu_seqlens[r + 1] - start;
+  if (len <= 0) return;
+  const int cols = a.vdim + 1;
+  const float* m_mem = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off + (size_t)a.heads * cols * a.dim + (size_t)h * cols;
+  float m = m_mem[0];      // (every column's copy is the same number)
+  const float bi = a.i_bias[h], bf = a.f_bias[h];
+  for (int t0 = 0; t0 < len; t0 += TP_WAVE) {
+    const bool mine = t0 + lane < len;
+    float gi = -INFINITY, gf = 0.f;      // (lanes past the run's end pass the sums along unchanged)
+    if (mine) {
+      const size_t row = (size_t)(start + t0 + lane) * a.stride;
+      gi = a.cap * tanhf((a.proj[row + a.i_col + h] + bi) / a.cap);
+      gf = m_logsigmoid(a.cap * tanhf((a.proj[row + a.f_col + h] + bf) / a.cap));
+    }
+    float F = gf;
+#pragma unroll
+    for (int d = 1; d < TP_WAVE; d *= 2) {
+      const float o = __shfl_up(F, d, TP_WAVE);
+      if (lane >= d) F += o;
+    }
+    float G = mine ? gi - F : -INFINITY;
+#pragma unroll
+    for (int d = 1; d < TP_WAVE; d *= 2) {
+      const float o = __shfl_up(G, d, TP_WAVE);
+      if (lane >= d) G = fmaxf(G, o);
+    }
+    const float m_new = F + fmaxf(m, G);
+    float m_prev = __shfl_up(m_new, 1, TP_WAVE);
+    if (lane == 0) m_prev = m;
+    if (mine) {
+      const size_t p = (size_t)(start + t0 + lane) * a.heads + h;
+      a.keep[p] = expf(gf + m_prev - m_new);
+      a.put[p] = expf(gi - m_new);
+      a.mrun[p] = m_new;
+    }
+    m = __shfl(m_new, TP_WAVE - 1, TP_WAVE);
+  }
+}
+
 template <int PER, int KS>
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
   constexpr int DP = PER * KS, CW = TP_WAVE / KS, CB = 4 * CW;
@@ -48,7 +95,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
   __shared__ __attribute__((aligned(16))) float qs[TC * DP];
   __shared__ __attribute__((aligned(16))) float kk[TC * DP];
   __shared__ float vs[TC * CB];
-  __shared__ float keep_s[TC], put_s[TC], m_s[TC + 1];
+  __shared__ float keep_s[TC], put_s[TC];
   const int r = blockIdx.x, h = blockIdx.y;
   const int start = a.cu_seqlens[r], len = a.cu_seqlens[r + 1] - start;
   if (len <= 0) return;
@@ -60,7 +107,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
 
   float* base = a.state + (size_t)a.state_slots[r] * a.state_stride + a.state_off;
   float* S_mem = base + ((size_t)h * cols + (col_ok ? j : 0)) * a.dim;
-  float* m_mem = base + (size_t)a.heads * cols * a.dim + (size_t)h * cols;
+  float* m_mem = base + (size_t)a.heads * cols * a.dim + (size_t)h * cols;   // (read by the kernel in front, written here)
   const bool vec = a.dim % 4 == 0 && ((uintptr_t)S_mem % 16) == 0;
   float S[PER];
 #pragma unroll
@@ -74,9 +121,6 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
       for (int c = 0; c < 4; ++c) S[e4 * 4 + c] = (col_ok && i + c < a.dim) ? S_mem[i + c] : 0.f;
     }
   }
-  // the running maximum as the block's first column holds it (every column's copy is the same number)
-  float m_run = m_mem[blockIdx.z * CB];
-
   const int q_col = a.q_col + h * a.dim, k_col = a.k_col + h * a.dim, v_col = a.v_col + h * a.vdim;
   float rq[NI], rk[NI], rv[NV], ri = 0.f, rf = 0.f;
   auto fetch = [&](int t0) {
@@ -102,9 +146,9 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
       rv[it] = v;
     }
     if (tid < TC && t0 + tid < len) {
-      const size_t row = (size_t)(start + t0 + tid) * a.stride;
-      ri = a.cap * tanhf((a.proj[row + a.i_col + h] + a.i_bias[h]) / a.cap);
-      rf = m_logsigmoid(a.cap * tanhf((a.proj[row + a.f_col + h] + a.f_bias[h]) / a.cap));
+      const size_t p = (size_t)(start + t0 + tid) * a.heads + h;
+      ri = a.put[p];
+      rf = a.keep[p];
     }
   };
   struct Tok {
@@ -145,7 +189,6 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
       const size_t row = (size_t)(start + t_run);
       if (is_n) {
         a.nq[row * a.heads + h] = rs;
-        a.mrun[row * a.heads + h] = m_s[t + 1];
       } else {
         a.num[row * out_width + (size_t)h * a.vdim + j] = rs;
       }
@@ -168,33 +211,11 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
       const int idx = it * 256 + tid;
       if (idx < TC * CB) vs[idx] = rv[it];
     }
-    if (wave == 0) {
-      // the chunk's gates: lanes 0..tc-1 hold a token each; lanes past the chunk's end pass the sums along unchanged
-      const bool mine = lane < tc;
-      float F = mine ? rf : 0.f;
-#pragma unroll
-      for (int d = 1; d < TC; d *= 2) {
-        const float o = __shfl_up(F, d, TP_WAVE);
-        if (lane >= d) F += o;
-      }
-      float G = mine ? ri - F : -INFINITY;
-#pragma unroll
-      for (int d = 1; d < TC; d *= 2) {
-        const float o = __shfl_up(G, d, TP_WAVE);
-        if (lane >= d) G = fmaxf(G, o);
-      }
-      const float m_new = F + fmaxf(m_run, G);
-      float m_prev = __shfl_up(m_new, 1, TP_WAVE);
-      if (lane == 0) m_prev = m_run;
-      if (mine) {
-        keep_s[lane] = expf(rf + m_prev - m_new);
-        put_s[lane] = expf(ri - m_new);
-        m_s[lane + 1] = m_new;
-      }
-      if (lane == 0) m_s[0] = m_run;
+    if (tid < TC) {
+      keep_s[tid] = rf;
+      put_s[tid] = ri;
     }
     __syncthreads();
-    m_run = m_s[tc];
     if (t0 + TC < len) fetch(t0 + TC);   // on its way while this chunk runs
     Tok A, B;
     take(A, 0);
@@ -218,7 +239,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(MlstmArgs a) {
         if (col_ok && i + c < a.dim) S_mem[i + c] = S[e4 * 4 + c];
     }
   }
-  if (ks == 0 && col_ok) m_mem[j] = m_run;
+  if (ks == 0 && col_ok) m_mem[j] = a.mrun[(size_t)(start + len - 1) * a.heads + h];
 }
 
 // out[t, out_col0 + h * vdim + d] = unit_rms(num[t, h, :] / (max(|nq|, e^(-m)) + 1e-6))[d] * w[h * vdim + d]
@@ -252,7 +273,7 @@ __global__ __launch_bounds__(256) void mlstm_out_kernel(const float* __restrict_
 }
 
 // proj columns from col0 on: [q (heads * dim) | k (heads * dim) | v (heads * vdim) | gate (heads * vdim) | i (heads) | f (heads)].
-// scratch: float32 [n * heads * (vdim + 2)].
+// scratch: float32 [n * heads * (vdim + 4)].
 extern "C" int tp_mlstm_scan(const float* proj, int stride, int col0, const float* i_bias, const float* f_bias, float cap,
                              float q_scale, float* state, size_t state_stride, size_t state_off, const int* cu_seqlens,
                              const int* state_slots, float* scratch, const float* norm_w, float eps, float scale, void* out,
@@ -288,9 +309,15 @@ extern "C" int tp_mlstm_scan(const float* proj, int stride, int col0, const floa
   a.num = scratch;
   a.nq = scratch + (size_t)n * heads * vdim;
   a.mrun = a.nq + (size_t)n * heads;
+  a.keep = a.mrun + (size_t)n * heads;
+  a.put = a.keep + (size_t)n * heads;
   a.heads = heads;
   a.dim = dim;
   a.vdim = vdim;
+  const long pairs = (long)n * heads;
+  TP_REQUIRE((pairs + 3) / 4 < 0x7fffffffL, "mlstm_scan: too many rows");
+  TP_REQUIRE(n_req <= 0x7fffffff / 1, "mlstm_scan: too many requests");
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(n_req, heads), dim3(64), 0, s, a);
   // PER key channels a lane (8 up to a key size of 128, then 16, then 32), KS lanes a column (a power of two)
   const int per = dim <= 128 ? 8 : (dim <= 256 ? 16 : 32);
   int ks = 1;
@@ -313,8 +340,6 @@ extern "C" int tp_mlstm_scan(const float* proj, int stride, int col0, const floa
   }
 #undef SCAN
   TP_CHECK_LAUNCH("mlstm_scan");
-  const long pairs = (long)n * heads;
-  TP_REQUIRE((pairs + 3) / 4 < 0x7fffffffL, "mlstm_scan: too many rows");
   const dim3 og((unsigned)((pairs + 3) / 4));
   if (out_dt == TP_F32)
     hipLaunchKernelGGL(mlstm_out_kernel<float>, og, dim3(256), 0, s, a.num, a.nq, a.mrun, norm_w, proj, stride, gate_col, eps, scale,

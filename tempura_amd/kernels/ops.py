@@ -1661,7 +1661,7 @@ def mlstm_scan(proj: torch.Tensor, col0: int, i_bias: torch.Tensor, f_bias: torc
     _i32(cu_seqlens, num_requests + 1, "cu_seqlens")
     _i32(state_slots, num_requests, "state_slots")
     _need(out.dim() == 2 and out.shape[0] == n and 0 <= out_col0 and out_col0 + heads * vdim <= out.shape[1], "mlstm_scan: output rows too short")
-    scratch = torch.empty((max(1, n * heads * (vdim + 2)),), dtype=torch.float32, device=proj.device)
+    scratch = torch.empty((max(2, n * heads * (vdim + 4)),), dtype=torch.float32, device=proj.device)
     _call("tp_mlstm_scan", _ptr(proj), proj.shape[1], int(col0), _ptr(i_bias), _ptr(f_bias), ctypes.c_float(cap), ctypes.c_float(q_scale),
           _ptr(state), ctypes.c_size_t(state.shape[1]), ctypes.c_size_t(state_off), _ptr(cu_seqlens), _ptr(state_slots), _ptr(scratch),
           _ptr(norm_weight), ctypes.c_float(eps), ctypes.c_float(scale), _ptr(out), _dt(out), out.shape[1], int(out_col0), n,
