@@ -87,17 +87,21 @@ class LatentMixer:
     dim: int
     vdim: int
     kv_rank: int
-    q_rank: int
+    q_rank: Optional[int]      # (None: the query latent's size is the tensors' own)
     scale: float
     kv_from: Optional[int] = None
 
     @classmethod
     def from_dict(cls, d, where):
-        return cls(_num(d, "heads", where), _num(d, "dim", where), _num(d, "vdim", where), _num(d, "kv_rank", where), _num(d, "q_rank", where),
+        dim = _num(d, "dim", where)
+        return cls(_num(d, "heads", where), dim, _num(d, "vdim", where) if d.get("vdim") is not None else dim, _num(d, "kv_rank", where),
+                   _num(d, "q_rank", where) if d.get("q_rank") is not None else None,
                    _num(d, "scale", where, float), None if d.get("kv_from") is None else _num(d, "kv_from", where, positive=False))
 
     def to_dict(self):
-        d = {"dim": self.dim, "heads": self.heads, "kv_rank": self.kv_rank, "q_rank": self.q_rank, "scale": self.scale, "vdim": self.vdim}
+        d = {"dim": self.dim, "heads": self.heads, "kv_rank": self.kv_rank, "scale": self.scale, "vdim": self.vdim}
+        if self.q_rank is not None:
+            d["q_rank"] = self.q_rank
         if self.kv_from is not None:
             d["kv_from"] = self.kv_from
         return d

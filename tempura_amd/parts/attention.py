@@ -533,7 +533,8 @@ class LatentCacheAttention(BranchMixer):
         self.head_dim = int(p["head_dim"])
         self.value_dim = int(p["value_dim"])
         self.latent_dim = int(p["latent_dim"])
-        self.query_rank = int(p["query_rank"])
+        #: the query latent's size: the configuration's, or (None) the checkpoint's own, known once the tensors are loaded
+        self.query_rank = int(p["query_rank"]) if p.get("query_rank") is not None else None
         self.scale = float(p["scale"])
         self.norm_eps = float(p["norm_eps"])
         self.window = p.get("window")
@@ -545,7 +546,8 @@ class LatentCacheAttention(BranchMixer):
     @classmethod
     def expected_weights(cls, spec, hidden_size):
         p, w = spec.params, spec.weights
-        H, D, Dv, L, Q = (int(p[k]) for k in ("num_heads", "head_dim", "value_dim", "latent_dim", "query_rank"))
+        H, D, Dv, L = (int(p[k]) for k in ("num_heads", "head_dim", "value_dim", "latent_dim"))
+        Q = int(p["query_rank"]) if p.get("query_rank") is not None else None      # (None: the checkpoint says it)
         out = {w["dq"]: WeightInfo((Q, hidden_size)), w["dq_norm"]: WeightInfo((Q,), "ones"), w["uq"]: WeightInfo((H * D, Q)),
                w["uk"]: WeightInfo((H * D, L)), w["uv"]: WeightInfo((H * Dv, L)), w["o"]: WeightInfo((hidden_size, H * Dv))}
         if p.get("own_latent", True):
@@ -562,6 +564,11 @@ class LatentCacheAttention(BranchMixer):
         w = self.spec.weights
         H, D, Dv, L = self.num_heads, self.head_dim, self.value_dim, self.latent_dim
         f64 = lambda name: get(w[name]).to(torch.float64)
+        dq = get(w["dq"])
+        if self.query_rank is None:
+            self.query_rank = int(dq.shape[0])
+        if get(w["uq"]).shape[1] != self.query_rank or dq.shape[0] != self.query_rank:
+            raise ValueError("latent_cache_attention: the two halves of the query projection disagree on its latent's size")
         uq, uk, uv, o = f64("uq").view(H, D, -1), f64("uk").view(H, D, L), f64("uv").view(H, Dv, L), f64("o").view(-1, H, Dv)
         # queries into the latent's space: rows h L .. (h + 1) L are W_uk[h]^T W_uq[h]
         q_fold = torch.einsum("hdl,hdq->hlq", uk, uq).reshape(H * L, -1)
@@ -569,7 +576,7 @@ class LatentCacheAttention(BranchMixer):
         # and the heads' sums over the latents back out: columns h L .. (h + 1) L are W_o[:, h] W_uv[h]
         o_fold = torch.einsum("whv,hvl->whl", o, uv).reshape(-1, H * L)
         self.dq_norm_w = self._to_device(get(w["dq_norm"]), torch.float32)
-        rows = [get(w["dq"])]
+        rows = [dq]
         if self.own_latent:
             rows.append(get(w["dkv"]))
             self.dkv_norm_w = self._to_device(get(w["dkv_norm"]), torch.float32)

@@ -366,3 +366,21 @@ def test_command_line_inspects_and_writes_random_folders(dirs, tmp_path, capsys)
     assert main(["random-model", "--config-json", str(path), "--out", str(tmp_path / "rnd"), "--std", "0.3"]) == 0
     model = load_model(str(tmp_path / "rnd"), "float32", "cpu")
     assert model.layers[3].mixer.norm_w.shape == (5,) and model.layers[2].mixer.w_q.shape == (11, 6)
+
+
+def test_a_size_the_configuration_leaves_out_is_the_tensors_own(tmp_path):
+    """Without `q_rank` the query latent's size comes from the checkpoint, without `vdim` values are as wide as keys,
+    without `max_positions` the position table has the rows it has."""
+    from tempura_amd.engine.runner import StepEntry
+    cfg = cases.config_json("one")
+    W = cases.make_weights("one")
+    del cfg["layers"][2]["mixer"]["q_rank"]
+    del cfg["layers"][1]["mixer"]["vdim"]
+    del cfg["max_positions"]
+    folder = cases.write_model("one", str(tmp_path / "lean"), weights=W, config=cfg)
+    runner = _runner(folder, 64)
+    assert runner.model.layers[2].mixer.query_rank == 6
+    toks = cases.tokens("one", 21, 3)
+    runner.add_request("r")
+    got = runner.step([StepEntry("r", toks, list(range(21)))])
+    assert plain.logit_error(got, plain.forward(cases.config_json("one"), W, toks)) < 1e-4
