@@ -365,8 +365,8 @@ def test_cutting_changes_rounding_only(dirs):
     lengths = cases.LENGTHS["wide"]
     runs = []
     for steps in (helpers.schedule_whole(lengths), helpers.schedule_portions(lengths, sizes=(2, 9, 33, 2, 16, 5)),
-                  helpers.schedule_mixed(lengths, 448, seed=3)):
-        runs.append(helpers.run_schedule(_runner(dirs["wide"], "float32", 448), reqs, steps))
+                  helpers.schedule_mixed(lengths, 512, seed=3)):
+        runs.append(helpers.run_schedule(_runner(dirs["wide"], "float32", 512), reqs, steps))
     for rid in reqs:
         for other in runs[1:]:
             assert plain.logit_error(other[rid], runs[0][rid]) < 1e-4, rid
